@@ -1,0 +1,232 @@
+"""The cache manager: pages of keys and values with a block table per request, in groups of cache
+entries with the same need, and slots of fixed-size state per request.
+
+Reference: data plane csrc/cache/kv_cache.cpp:113-148 (one tensor per layer, here K and V apart,
+each [pages, nkv, page, d]); control plane python/infinilm/llm/cache_manager.py:158-191 (pages for
+a prompt), :317-328 (a new page iff the new token opens one), :330-348 (giving back); fixed-size
+state csrc/cache/mamba_cache.cpp:8-47 and cache_manager.py:33-68 (row 0 is the zero state, rows
+from a free list).  Differences by design: pages are reserved portion by portion instead of for
+the whole prompt at admission, go straight back to the free list when a request ends or a window
+has passed them, and cache entries whose mixers keep all keys and those that keep a window form
+groups with page pools and block tables of their own.
+
+The control plane (this class) holds no GPU state beyond the tensors it allocates; it can be built
+with device="meta" or "cpu" and exercised without a GPU.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from .needs import FixedState, PagedKV
+from .pages import CacheError, OutOfPages, PagePool
+
+
+@dataclass
+class _Group:
+    """Cache entries that share a page-id space and a block table per request."""
+    window: int
+    entries: List[int]
+    pool: PagePool
+
+
+@dataclass
+class _Request:
+    length: int = 0                      # tokens whose keys are in the cache
+    reserved: int = 0                    # tokens pages are held for (>= length)
+    tables: List[List[int]] = field(default_factory=list)   # per group: logical page -> page id, -1 = given back
+    state_slot: int = 0
+    fresh: bool = True                   # no state written yet: reads start from the zero row
+
+
+class KVView:
+    """What a mixer's forward gets for a paged entry."""
+    __slots__ = ("k", "v", "page_size", "block_tables", "slots", "window")
+
+    def __init__(self, k, v, page_size, block_tables, slots, window):
+        self.k, self.v, self.page_size, self.block_tables, self.slots, self.window = k, v, page_size, block_tables, slots, window
+
+
+class StateView:
+    """What a mixer's forward gets for a fixed-size state entry: the pool [slots, *shape], the row
+    each request reads at the start of the step (0 = zeros) and the row it writes at the end."""
+    __slots__ = ("pool", "state_in", "state_out")
+
+    def __init__(self, pool, state_in, state_out):
+        self.pool, self.state_in, self.state_out = pool, state_in, state_out
+
+
+class CacheManager:
+    def __init__(self, needs: Sequence, page_size: int, num_pages: int, max_requests: int,
+                 dtype: torch.dtype, device, num_pages_per_group: Optional[Dict[int, int]] = None):
+        if page_size <= 0:
+            raise CacheError(f"page size must be positive, got {page_size}")
+        self.page_size = int(page_size)
+        self.max_requests = int(max_requests)
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.needs = list(needs)
+        self.groups: List[_Group] = []
+        self.group_of_entry: Dict[int, int] = {}
+        by_window: Dict[int, int] = {}
+        for e, need in enumerate(self.needs):
+            if isinstance(need, PagedKV):
+                if need.window not in by_window:
+                    n = (num_pages_per_group or {}).get(need.window, num_pages)
+                    by_window[need.window] = len(self.groups)
+                    self.groups.append(_Group(need.window, [], PagePool(n)))
+                g = by_window[need.window]
+                self.groups[g].entries.append(e)
+                self.group_of_entry[e] = g
+        # data plane
+        self.k: Dict[int, torch.Tensor] = {}
+        self.v: Dict[int, torch.Tensor] = {}
+        self.state: Dict[int, torch.Tensor] = {}
+        for e, need in enumerate(self.needs):
+            if isinstance(need, PagedKV):
+                n = self.groups[self.group_of_entry[e]].pool.num_pages
+                shape = (n, need.num_kv_heads, self.page_size, need.head_dim)
+                self.k[e] = torch.zeros(shape, dtype=dtype, device=self.device)
+                self.v[e] = torch.zeros(shape, dtype=dtype, device=self.device)
+            elif isinstance(need, FixedState):
+                self.state[e] = torch.zeros((self.max_requests + 1,) + tuple(need.shape),
+                                            dtype=need.dtype or torch.float32, device=self.device)
+            elif need is not None:
+                raise CacheError(f"cache entry {e}: unknown need {need!r}")
+        # state slots: row 0 is the permanent zero state
+        self._free_slots = list(range(self.max_requests, 0, -1))
+        self.requests: Dict[object, _Request] = {}
+
+    # ---- sizes ----------------------------------------------------------------------------------
+    def bytes_per_token(self) -> int:
+        total = 0
+        for e, need in enumerate(self.needs):
+            if isinstance(need, PagedKV):
+                total += 2 * need.num_kv_heads * need.head_dim * self.k[e].element_size()
+        return total
+
+    def free_pages(self, group: int = 0) -> int:
+        return self.groups[group].pool.num_free if self.groups else 0
+
+    def total_pages(self, group: int = 0) -> int:
+        return self.groups[group].pool.num_pages if self.groups else 0
+
+    def stats(self) -> dict:
+        return {"requests": len(self.requests),
+                "groups": [{"window": g.window, "entries": len(g.entries), "pages": g.pool.num_pages,
+                            "free": g.pool.num_free, "high_water": g.pool.high_water} for g in self.groups],
+                "state_slots_free": len(self._free_slots)}
+
+    # ---- requests -------------------------------------------------------------------------------
+    def admit(self, req_id) -> None:
+        if req_id in self.requests:
+            raise CacheError(f"request {req_id!r} is already admitted")
+        if not self._free_slots:
+            raise CacheError(f"no state slot free for request {req_id!r} ({self.max_requests} requests at most)")
+        r = _Request(tables=[[] for _ in self.groups], state_slot=self._free_slots.pop())
+        self.requests[req_id] = r
+
+    def has(self, req_id) -> bool:
+        return req_id in self.requests
+
+    def length(self, req_id) -> int:
+        return self.requests[req_id].length
+
+    def _first_needed_page(self, group: _Group, first_query_pos: int) -> int:
+        if group.window <= 0:
+            return 0
+        lo = max(0, first_query_pos - group.window + 1)
+        return lo // self.page_size
+
+    def pages_needed(self, req_id, n_new: int) -> List[int]:
+        """Pages each group would have to take so that `n_new` more tokens fit."""
+        r = self.requests[req_id]
+        upto = r.length + n_new
+        out = []
+        for g, table in zip(self.groups, r.tables):
+            want = -(-upto // self.page_size)
+            out.append(max(0, want - len(table)))
+        return out
+
+    def can_reserve(self, req_id, n_new: int) -> bool:
+        return all(n <= g.pool.num_free for n, g in zip(self.pages_needed(req_id, n_new), self.groups))
+
+    def reserve(self, req_id, n_new: int) -> None:
+        """Take the pages for `n_new` tokens after the cached ones in every group, or OutOfPages
+        with nothing taken."""
+        r = self.requests[req_id]
+        if n_new <= 0:
+            raise CacheError(f"reserve of {n_new} tokens")
+        need = self.pages_needed(req_id, n_new)
+        for n, g in zip(need, self.groups):
+            if n > g.pool.num_free:
+                raise OutOfPages(f"request {req_id!r}: {n} pages needed for {n_new} tokens after {r.length}, "
+                                 f"{g.pool.num_free} free of {g.pool.num_pages} (window {g.window})")
+        for n, g, table in zip(need, self.groups, r.tables):
+            table.extend(g.pool.take(n))
+        r.reserved = max(r.reserved, r.length + n_new)
+
+    def commit(self, req_id, n_new: int) -> None:
+        """`n_new` tokens have been written; give back the pages a window has passed."""
+        r = self.requests[req_id]
+        if r.length + n_new > r.reserved:
+            raise CacheError(f"request {req_id!r}: commit of {n_new} tokens beyond what was reserved")
+        r.length += n_new
+        r.fresh = False
+        for g, table in zip(self.groups, r.tables):
+            first = self._first_needed_page(g, r.length)  # the next query sits at position `length`
+            for i in range(min(first, len(table))):
+                if table[i] >= 0:
+                    g.pool.give_back([table[i]])
+                    table[i] = -1
+
+    def slot_of(self, req_id, group: int, position: int) -> int:
+        """slot = page_id * page_size + offset (cache_manager.py:186-191)."""
+        table = self.requests[req_id].tables[group]
+        page = table[position // self.page_size]
+        if page < 0:
+            raise CacheError(f"request {req_id!r}: position {position} lies on a page already given back")
+        return page * self.page_size + position % self.page_size
+
+    def table(self, req_id, group: int) -> List[int]:
+        return self.requests[req_id].tables[group]
+
+    def state_rows(self, req_id):
+        """(row read at the start of the step, row written at its end)."""
+        r = self.requests[req_id]
+        return (0 if r.fresh else r.state_slot), r.state_slot
+
+    def release(self, req_id) -> None:
+        """The request is over (or preempted): all its pages and its slot go back."""
+        r = self.requests.pop(req_id, None)
+        if r is None:
+            raise CacheError(f"request {req_id!r} is not admitted (released twice?)")
+        for g, table in zip(self.groups, r.tables):
+            g.pool.give_back([p for p in table if p >= 0])
+        self._free_slots.append(r.state_slot)
+
+    def check(self) -> None:
+        """No page lost, none held twice: the pages in the block tables are exactly the held ones."""
+        for gi, g in enumerate(self.groups):
+            g.pool.check()
+            held = [p for r in self.requests.values() for p in r.tables[gi] if p >= 0]
+            if len(held) != len(set(held)):
+                raise CacheError(f"group {gi}: a page is in two block tables")
+            if len(held) != g.pool.num_held:
+                raise CacheError(f"group {gi}: {g.pool.num_held} pages held, {len(held)} in block tables")
+        slots = [r.state_slot for r in self.requests.values()]
+        if len(set(slots)) != len(slots) or set(slots) & set(self._free_slots) or 0 in slots:
+            raise CacheError("state slots are inconsistent")
+
+    # ---- what a layer sees --------------------------------------------------------------------
+    def view(self, entry: int, batch, writes: bool):
+        need = self.needs[entry]
+        if isinstance(need, PagedKV):
+            g = self.group_of_entry[entry]
+            return KVView(self.k[entry], self.v[entry], self.page_size, batch.block_tables[g],
+                          batch.slots[g] if writes else None, need.window)
+        if isinstance(need, FixedState):
+            return StateView(self.state[entry], batch.state_in, batch.state_out)
+        return None

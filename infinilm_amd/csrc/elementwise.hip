@@ -1,0 +1,212 @@
+// Memory-bound kernels of the step: embedding gather, residual add + RMSNorm, rotation + cache
+// write, SwiGLU, row gather.  All arithmetic is float; T is the activation type (float or bf16).
+#include <stdarg.h>
+
+#include "common.h"
+
+static thread_local char g_err[1024] = {0};
+
+extern "C" const char* ilm_last_error() { return g_err; }
+
+void ilm_set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+// ------------------------------------------------------------------------------------------
+// embedding: r[t, :] = scale * E[ids[t], :]   (residual stream, float)
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(float* __restrict__ r, const int* __restrict__ ids,
+                             const T* __restrict__ table, int H, float scale) {
+    const int t = blockIdx.x;
+    const T* row = table + (size_t)ids[t] * H;
+    float* out = r + (size_t)t * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) out[j] = scale * to_f32(row[j]);
+}
+
+extern "C" int ilm_embed(void* r, const void* ids, const void* table, int T_, int H, int V,
+                         float scale, int dtype, hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T_, H, V);
+    if (dtype == ILM_DTYPE_F32)
+        embed_kernel<float><<<T_, 256, 0, stream>>>((float*)r, (const int*)ids, (const float*)table, H, scale);
+    else if (dtype == ILM_DTYPE_BF16)
+        embed_kernel<bf16><<<T_, 256, 0, stream>>>((float*)r, (const int*)ids, (const bf16*)table, H, scale);
+    else
+        ILM_REQUIRE(false, "embed: unknown dtype %d", dtype);
+    ILM_LAUNCH_CHECK("embed");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// r += alpha * h ; x = r / sqrt(mean(r^2) + eps) * w
+// One block per row.  The sum of squares is reduced in an order that depends on H only, so a
+// row's result does not depend on what else is in the batch.
+// ------------------------------------------------------------------------------------------
+template <typename T, typename WT>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_kernel(T* __restrict__ x, float* __restrict__ r, const T* __restrict__ h,
+                   const WT* __restrict__ w, int H, float alpha, float eps) {
+    __shared__ float red[4];
+    const size_t base = (size_t)blockIdx.x * H;
+    float ss = 0.f;
+    if (h != nullptr) {
+        for (int j = threadIdx.x; j < H; j += 256) {
+            float v = r[base + j] + alpha * to_f32(h[base + j]);
+            r[base + j] = v;
+            ss += v * v;
+        }
+    } else {
+        for (int j = threadIdx.x; j < H; j += 256) {
+            float v = r[base + j];
+            ss += v * v;
+        }
+    }
+    const float tot = block_sum<4>(ss, red);
+    const float rstd = 1.0f / sqrtf(tot / (float)H + eps);
+    for (int j = threadIdx.x; j < H; j += 256)
+        x[base + j] = from_f32<T>(r[base + j] * rstd * to_f32(w[j]));
+}
+
+extern "C" int ilm_add_rmsnorm(void* x, void* r, const void* h, const void* w, int rows, int H,
+                               float alpha, float eps, int dtype, int w_dtype,
+                               hipStream_t stream) {
+    ILM_REQUIRE(rows > 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", rows, H);
+#define NORM_CASE(T, WT)                                                                      \
+    add_rmsnorm_kernel<T, WT><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const T*)h,        \
+                                                        (const WT*)w, H, alpha, eps)
+    if (dtype == ILM_DTYPE_F32 && w_dtype == ILM_DTYPE_F32) NORM_CASE(float, float);
+    else if (dtype == ILM_DTYPE_BF16 && w_dtype == ILM_DTYPE_BF16) NORM_CASE(bf16, bf16);
+    else if (dtype == ILM_DTYPE_BF16 && w_dtype == ILM_DTYPE_F32) NORM_CASE(bf16, float);
+    else if (dtype == ILM_DTYPE_F32 && w_dtype == ILM_DTYPE_BF16) NORM_CASE(float, bf16);
+    else ILM_REQUIRE(false, "add_rmsnorm: unknown dtypes %d %d", dtype, w_dtype);
+#undef NORM_CASE
+    ILM_LAUNCH_CHECK("add_rmsnorm");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Rotation of q and k in place (pairs (i, i + rd/2), tables cos/sin [max_pos, rd/2] float), and
+// the write of the rotated k and of v into the paged cache [pages, nkv, page, d] at
+// slot = page_id * page + offset.  One block of 64 threads per (token, head slot); head slots
+// are nh query heads, then nkv key heads, then nkv value heads, as they lie in the qkv row.
+// slot < 0: nothing is written to the cache for that token.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(64)
+rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ pos, const float* __restrict__ cosT,
+                    const float* __restrict__ sinT, T* __restrict__ kc, T* __restrict__ vc,
+                    const int* __restrict__ slots, int nh, int nkv, int d, int rd, int row_stride,
+                    int page) {
+    const int t = blockIdx.x, hs = blockIdx.y;
+    T* p = qkv + (size_t)t * row_stride + (size_t)hs * d;
+    const int half = rd >> 1;
+    const bool is_v = hs >= nh + nkv;
+    const bool is_k = !is_v && hs >= nh;
+    T* dst = nullptr;
+    if ((is_k || is_v) && slots != nullptr) {
+        const int slot = slots[t];
+        if (slot >= 0) {
+            const int kvh = is_k ? hs - nh : hs - nh - nkv;
+            const size_t off = (((size_t)(slot / page) * nkv + kvh) * page + (slot % page)) * d;
+            dst = (is_k ? kc : vc) + off;
+        }
+    }
+    if (is_v) {
+        if (dst != nullptr)
+            for (int i = threadIdx.x; i < d; i += 64) dst[i] = p[i];
+        return;
+    }
+    const float* c = cosT + (size_t)pos[t] * half;
+    const float* s = sinT + (size_t)pos[t] * half;
+    for (int i = threadIdx.x; i < half; i += 64) {
+        const float a = to_f32(p[i]), b = to_f32(p[i + half]);
+        const T ra = from_f32<T>(a * c[i] - b * s[i]);
+        const T rb = from_f32<T>(b * c[i] + a * s[i]);
+        p[i] = ra;
+        p[i + half] = rb;
+        if (dst != nullptr) {
+            dst[i] = ra;
+            dst[i + half] = rb;
+        }
+    }
+    if (dst != nullptr)
+        for (int i = rd + threadIdx.x; i < d; i += 64) dst[i] = p[i];
+}
+
+extern "C" int ilm_rope_kvwrite(void* qkv, const void* pos, const void* cosT, const void* sinT,
+                                void* kc, void* vc, const void* slots, int T_, int nh, int nkv,
+                                int d, int rd, int row_stride, int page, int dtype,
+                                hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && nh > 0 && nkv >= 0 && d > 0, "rope_kvwrite: bad sizes");
+    ILM_REQUIRE(rd >= 0 && rd <= d && rd % 2 == 0, "rope_kvwrite: rotary dim %d does not fit head dim %d", rd, d);
+    ILM_REQUIRE(row_stride >= (nh + 2 * nkv) * d, "rope_kvwrite: row stride %d too small", row_stride);
+    ILM_REQUIRE(slots == nullptr || page > 0, "rope_kvwrite: page size %d", page);
+    dim3 grid(T_, nh + 2 * nkv);
+    if (dtype == ILM_DTYPE_F32)
+        rope_kvwrite_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, (const int*)pos, (const float*)cosT,
+                                                           (const float*)sinT, (float*)kc, (float*)vc,
+                                                           (const int*)slots, nh, nkv, d, rd, row_stride, page);
+    else if (dtype == ILM_DTYPE_BF16)
+        rope_kvwrite_kernel<bf16><<<grid, 64, 0, stream>>>((bf16*)qkv, (const int*)pos, (const float*)cosT,
+                                                          (const float*)sinT, (bf16*)kc, (bf16*)vc,
+                                                          (const int*)slots, nh, nkv, d, rd, row_stride, page);
+    else
+        ILM_REQUIRE(false, "rope_kvwrite: unknown dtype %d", dtype);
+    ILM_LAUNCH_CHECK("rope_kvwrite");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// act[t, i] = silu(gu[t, i]) * gu[t, I + i]   (gate is the first half of the fused projection)
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, int I, int gu_stride) {
+    const int t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= I) return;
+    const float g = to_f32(gu[(size_t)t * gu_stride + i]);
+    const float u = to_f32(gu[(size_t)t * gu_stride + I + i]);
+    out[(size_t)t * I + i] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int ilm_swiglu(void* out, const void* gu, int T_, int I, int gu_stride, int dtype,
+                          hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && I > 0 && gu_stride >= 2 * I, "swiglu: bad sizes T=%d I=%d stride=%d", T_, I, gu_stride);
+    ILM_REQUIRE(T_ <= 65535, "swiglu: at most 65535 rows a call, got %d", T_);
+    dim3 grid((I + 255) / 256, T_);
+    if (dtype == ILM_DTYPE_F32)
+        swiglu_kernel<float><<<grid, 256, 0, stream>>>((float*)out, (const float*)gu, I, gu_stride);
+    else if (dtype == ILM_DTYPE_BF16)
+        swiglu_kernel<bf16><<<grid, 256, 0, stream>>>((bf16*)out, (const bf16*)gu, I, gu_stride);
+    else
+        ILM_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+    ILM_LAUNCH_CHECK("swiglu");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// out[i, :] = in[idx[i], :]
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void gather_rows_kernel(T* __restrict__ out, const T* __restrict__ in,
+                                   const int* __restrict__ idx, int H) {
+    const T* src = in + (size_t)idx[blockIdx.x] * H;
+    T* dst = out + (size_t)blockIdx.x * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = src[j];
+}
+
+extern "C" int ilm_gather_rows(void* out, const void* in, const void* idx, int n, int H, int dtype,
+                               hipStream_t stream) {
+    ILM_REQUIRE(n > 0 && H > 0, "gather_rows: bad sizes n=%d H=%d", n, H);
+    if (dtype == ILM_DTYPE_F32)
+        gather_rows_kernel<float><<<n, 256, 0, stream>>>((float*)out, (const float*)in, (const int*)idx, H);
+    else if (dtype == ILM_DTYPE_BF16)
+        gather_rows_kernel<bf16><<<n, 256, 0, stream>>>((bf16*)out, (const bf16*)in, (const int*)idx, H);
+    else
+        ILM_REQUIRE(false, "gather_rows: unknown dtype %d", dtype);
+    ILM_LAUNCH_CHECK("gather_rows");
+    return 0;
+}

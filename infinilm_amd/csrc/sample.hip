@@ -1,0 +1,201 @@
+// Sampling from rows of float logits: argmax, and temperature / top-k / top-p with an inverse CDF.
+//
+// Definition: temperature == 0 or top_k == 1 -> the first index of the maximum.  Otherwise
+// e_i = exp((l_i - max) / temperature); keep the top_k largest logits (0 or >= V keeps all; ties
+// with the k-th value are kept); among those keep the fewest largest whose mass reaches top_p of
+// the kept mass (ties kept); the token is the first index, in vocabulary order over the kept set,
+// whose running mass exceeds u * (kept mass), u in [0, 1) supplied by the host per row.
+// Thresholds are found by building the k-th largest value bit by bit over an order-preserving
+// integer image of the floats, so no sort and no scratch memory is needed; one block per row.
+#include "common.h"
+
+#define SB 1024
+#define SNW (SB / 64)
+
+__device__ __forceinline__ uint32_t okey(float f) {
+    uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__device__ __forceinline__ void better(float& bv, int& bi, float v, int i) {
+    if (v > bv || (v == bv && i < bi)) {
+        bv = v;
+        bi = i;
+    }
+}
+
+// argmax of one row by the whole block (first index on ties); result valid in every thread
+__device__ int block_argmax(const float* __restrict__ row, int V, float* sv, int* si, float* out_max) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += SB) better(bv, bi, row[i], i);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        float ov = __shfl_xor(bv, o, 64);
+        int oi = __shfl_xor(bi, o, 64);
+        better(bv, bi, ov, oi);
+    }
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) {
+        sv[w] = bv;
+        si[w] = bi;
+    }
+    __syncthreads();
+    bv = sv[0];
+    bi = si[0];
+    for (int i = 1; i < SNW; ++i) better(bv, bi, sv[i], si[i]);
+    if (bi == 0x7fffffff) bi = 0;  // a row of NaN
+    *out_max = bv;
+    return bi;
+}
+
+__global__ void __launch_bounds__(SB)
+argmax_kernel(int* __restrict__ out, const float* __restrict__ logits, int V, int stride) {
+    __shared__ float sv[SNW];
+    __shared__ int si[SNW];
+    float mx;
+    const int bi = block_argmax(logits + (size_t)blockIdx.x * stride, V, sv, si, &mx);
+    if (threadIdx.x == 0) out[blockIdx.x] = bi;
+}
+
+extern "C" int ilm_argmax(void* out, const void* logits, int n, int V, int stride,
+                          hipStream_t stream) {
+    ILM_REQUIRE(n > 0 && V > 0 && stride >= V, "argmax: bad sizes n=%d V=%d stride=%d", n, V, stride);
+    argmax_kernel<<<n, SB, 0, stream>>>((int*)out, (const float*)logits, V, stride);
+    ILM_LAUNCH_CHECK("argmax");
+    return 0;
+}
+
+__device__ __forceinline__ float block_sum_f(float v, float* red) { return block_sum<SNW>(v, red); }
+
+__device__ __forceinline__ int block_sum_i(int v, int* red) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    int t = 0;
+#pragma unroll
+    for (int i = 0; i < SNW; ++i) t += red[i];
+    return t;
+}
+
+__global__ void __launch_bounds__(SB)
+sample_kernel(int* __restrict__ out, const float* __restrict__ logits, const float* __restrict__ temperature,
+              const int* __restrict__ top_k, const float* __restrict__ top_p,
+              const float* __restrict__ uniform, int V, int stride) {
+    __shared__ float sv[SNW];
+    __shared__ int si[SNW];
+    __shared__ float redf[SNW];
+    __shared__ int redi[SNW];
+    __shared__ float wave_tot[SNW];
+    __shared__ int claim;
+    __shared__ int last_kept;
+    const int r = blockIdx.x;
+    const float* row = logits + (size_t)r * stride;
+    const float temp = temperature[r];
+    const int k = top_k[r];
+    const float pp = top_p[r];
+    float mx;
+    const int amax = block_argmax(row, V, sv, si, &mx);
+    if (temp == 0.0f || k == 1) {
+        if (threadIdx.x == 0) out[r] = amax;
+        return;
+    }
+    const float inv_t = 1.0f / temp;
+
+    // threshold of the top-k: the k-th largest key
+    uint32_t tau = 0u;
+    if (k > 0 && k < V) {
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = tau | (1u << bit);
+            int c = 0;
+            for (int i = threadIdx.x; i < V; i += SB) c += okey(row[i]) >= cand;
+            if (block_sum_i(c, redi) >= k) tau = cand;
+        }
+    }
+    // threshold of the top-p within the kept set
+    if (pp < 1.0f) {
+        float sk = 0.f;
+        for (int i = threadIdx.x; i < V; i += SB)
+            if (okey(row[i]) >= tau) sk += expf((row[i] - mx) * inv_t);
+        sk = block_sum_f(sk, redf);
+        const float need = pp * sk;
+        uint32_t tp = 0u;
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = tp | (1u << bit);
+            const uint32_t thr = cand > tau ? cand : tau;
+            float ms = 0.f;
+            for (int i = threadIdx.x; i < V; i += SB)
+                if (okey(row[i]) >= thr) ms += expf((row[i] - mx) * inv_t);
+            if (block_sum_f(ms, redf) >= need) tp = cand;
+        }
+        if (tp > tau) tau = tp;
+    }
+    // inverse CDF in vocabulary order over the kept set
+    const int chunk = (V + SB - 1) / SB;
+    const int i0 = threadIdx.x * chunk;
+    const int i1 = (i0 + chunk < V) ? i0 + chunk : V;
+    float local = 0.f;
+    int my_last = -1;
+    for (int i = i0; i < i1; ++i)
+        if (okey(row[i]) >= tau) {
+            local += expf((row[i] - mx) * inv_t);
+            my_last = i;
+        }
+    // inclusive scan of `local` over the block
+    float incl = local;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float n = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += n;
+    }
+    if (threadIdx.x == 0) {
+        claim = 0x7fffffff;
+        last_kept = -1;
+    }
+    __syncthreads();
+    if (lane == 63) wave_tot[w] = incl;
+    __syncthreads();
+    float before = 0.f, total = 0.f;
+    for (int i = 0; i < SNW; ++i) {
+        if (i < w) before += wave_tot[i];
+        total += wave_tot[i];
+    }
+    incl += before;
+    const float target = uniform[r] * total;
+    if (local > 0.f && target < incl) atomicMin(&claim, (int)threadIdx.x);
+    if (my_last >= 0) atomicMax(&last_kept, my_last);
+    __syncthreads();
+    if (claim == 0x7fffffff) {
+        if (threadIdx.x == 0) out[r] = last_kept >= 0 ? last_kept : amax;
+        return;
+    }
+    if ((int)threadIdx.x == claim) {
+        float cum = incl - local;
+        int pick = my_last;
+        for (int i = i0; i < i1; ++i)
+            if (okey(row[i]) >= tau) {
+                cum += expf((row[i] - mx) * inv_t);
+                if (target < cum) {
+                    pick = i;
+                    break;
+                }
+            }
+        out[r] = pick;
+    }
+}
+
+extern "C" int ilm_sample(void* out, const void* logits, const void* temperature, const void* top_k,
+                          const void* top_p, const void* uniform, int n, int V, int stride,
+                          hipStream_t stream) {
+    ILM_REQUIRE(n > 0 && V > 0 && stride >= V, "sample: bad sizes n=%d V=%d stride=%d", n, V, stride);
+    sample_kernel<<<n, SB, 0, stream>>>((int*)out, (const float*)logits, (const float*)temperature,
+                                        (const int*)top_k, (const float*)top_p, (const float*)uniform,
+                                        V, stride);
+    ILM_LAUNCH_CHECK("sample");
+    return 0;
+}

@@ -1,0 +1,61 @@
+"""From a model folder to a built model with its weights, and to a step runner with a cache."""
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from ..cache import CacheManager
+from ..config.registry import load_model_config
+from ..weights.loader import load_weights
+from .model import CausalLM
+from .step import StepRunner
+
+_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "fp32": torch.float32, "bf16": torch.bfloat16,
+           torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
+
+
+def resolve_dtype(dtype, config_dtype: Optional[str]) -> torch.dtype:
+    """`dtype` given wins; else config.json's `dtype`/`torch_dtype` (csrc/config/model_config.cpp:28-39).
+    float16 checkpoints run in bfloat16: the kernels here take float32 and bfloat16."""
+    if dtype is None:
+        if config_dtype is None:
+            raise ValueError("No dtype or torch_dtype found in config, and none was given")
+        dtype = "bfloat16" if config_dtype == "float16" else config_dtype
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"Unsupported dtype string: {dtype}") from None
+
+
+def require_gpu(device) -> torch.device:
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError("infinilm_amd runs on an AMD GPU only (device 'cuda:N' under ROCm); "
+                           "there is no CPU path")
+    return device
+
+
+def build_model(model_dir_or_config, dtype=None, device="cuda:0") -> CausalLM:
+    """The model for a config.json (a folder or its parsed dict), parameters uninitialised."""
+    arch, cfg = load_model_config(model_dir_or_config)
+    spec = arch.build_spec(cfg)
+    dt = resolve_dtype(dtype, getattr(cfg, "dtype", None))
+    model = CausalLM(spec, dt, device)
+    model.config = cfg
+    return model
+
+
+def load_model(model_dir: str, dtype=None, device="cuda:0") -> CausalLM:
+    device = require_gpu(device)
+    from ..csrc import lib
+    lib.load()  # compile the kernels first if need be, and fail early without them
+    model = build_model(model_dir, dtype, device)
+    load_weights(model, model_dir)
+    return model
+
+
+def make_runner(model: CausalLM, num_pages: int, page_size: int, max_requests: int) -> StepRunner:
+    cache = CacheManager(model.cache_needs, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
+                         dtype=model.dtype, device=model.device)
+    return StepRunner(model, cache)

@@ -1,0 +1,212 @@
+"""The step function: a batch of (request, its next tokens) in, logits at the wanted places out.
+
+A step runs only the tokens it is given, as one flattened batch, from the cache that earlier steps
+left: portions of prompts beside single decoded tokens, cut anywhere.  Reference for the tensors a
+step carries: python/infinilm/processors/basic_llm_processor.py:161-263 (token ids, positions,
+lengths, offsets, block tables padded with -1, slot mapping) and csrc/engine/infer_engine.cpp:187-254
+(copy to the device once per step).  Unlike the reference, positions are derived from the cache
+manager's record of each request, all metadata goes to the device in one copy, and there is one
+attention contract for every kind of segment (the reference switches kernels by `T != R`,
+csrc/layers/attention/backends/paged_attn.cpp:36-37).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager
+
+
+@dataclass
+class StepEntry:
+    """A request's next tokens and the places among them whose logits are wanted."""
+    req_id: object
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+class StepBatch:
+    """Device-side metadata of one step (all int32), plus a few host-side facts kernels dispatch on."""
+
+    def __init__(self):
+        self.T = 0                      # tokens in the step
+        self.R = 0                      # requests in the step
+        self.token_ids = None           # [T]
+        self.positions = None           # [T] absolute position of each token in its request
+        self.seg_of_token = None        # [T] index of the token's request in this batch
+        self.seg_offsets = None         # [R+1] prefix sums of new-token counts
+        self.start_pos = None           # [R] tokens cached before this step
+        self.total_lens = None          # [R] tokens cached after this step
+        self.want_rows = None           # [num_wanted] rows of the flattened batch
+        self.state_in = None            # [R] state row read at the start (0 = zeros)
+        self.state_out = None           # [R] state row written at the end
+        self.block_tables: List = []    # per group [R, max_blocks], -1 padded
+        self.slots: List = []           # per group [T] slot of each new token
+        self.num_wanted = 0
+        self.wants_all_rows = False
+        self.max_q_len = 0
+        self.max_total_len = 0
+        self.max_position = 0
+        self.all_decode = False
+        # host copies for parts that plan on the host
+        self.h_seg_offsets: Optional[np.ndarray] = None
+        self.h_start_pos: Optional[np.ndarray] = None
+        self.taps: Optional[dict] = None
+
+
+class StepRunner:
+    """Owns the model and the cache manager; `step()` is the one function that advances requests."""
+
+    def __init__(self, model, cache: CacheManager):
+        self.model = model
+        self.cache = cache
+        self.device = model.device
+        self._pinned: Optional[torch.Tensor] = None
+        self._copy_done: Optional[torch.cuda.Event] = None
+        self.steps = 0
+        self.tokens = 0
+
+    # ---- batch building -----------------------------------------------------------------------
+    def _stage(self, n: int) -> torch.Tensor:
+        if self._copy_done is not None:
+            self._copy_done.synchronize()
+        if self._pinned is None or self._pinned.numel() < n:
+            self._pinned = torch.empty((max(n, 4096) * 2,), dtype=torch.int32, pin_memory=self.device.type == "cuda")
+        return self._pinned[:n]
+
+    def build_batch(self, entries: Sequence[StepEntry]) -> StepBatch:
+        """Reserves pages for every entry (all or nothing) and lays the step's metadata out."""
+        cache = self.cache
+        V = self.model.spec.vocab_size
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        seen = set()
+        for e in entries:
+            if e.req_id in seen:
+                raise ValueError(f"request {e.req_id!r} appears twice in one step")
+            seen.add(e.req_id)
+            if len(e.tokens) == 0:
+                raise ValueError(f"request {e.req_id!r} brings no tokens")
+            n = len(e.tokens)
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise ValueError(f"request {e.req_id!r}: wanted place {w} is outside its {n} tokens")
+            for t in e.tokens:
+                if not 0 <= t < V:
+                    raise ValueError(f"request {e.req_id!r}: token id {t} is outside the vocabulary of {V}")
+            if cache.length(e.req_id) + n > self.model.spec.max_positions:
+                raise ValueError(f"request {e.req_id!r}: {cache.length(e.req_id) + n} tokens exceed the model's "
+                                 f"{self.model.spec.max_positions} positions")
+        reserved = []
+        try:
+            for e in entries:
+                cache.reserve(e.req_id, len(e.tokens))
+                reserved.append(e)
+        except Exception:
+            # pages taken for earlier entries of this step stay with their requests (they will be
+            # used by the same tokens later); nothing is half-written
+            raise
+
+        R = len(entries)
+        lens = np.array([len(e.tokens) for e in entries], dtype=np.int64)
+        T = int(lens.sum())
+        start = np.array([cache.length(e.req_id) for e in entries], dtype=np.int64)
+        offsets = np.zeros(R + 1, dtype=np.int64)
+        np.cumsum(lens, out=offsets[1:])
+        G = len(cache.groups)
+        ps = cache.page_size
+        max_blocks = [max(1, max(len(cache.table(e.req_id, g)) for e in entries)) for g in range(G)]
+        n_want = sum(len(e.want) for e in entries)
+
+        # layout of the one int32 buffer
+        sizes = [("token_ids", T), ("positions", T), ("seg_of_token", T), ("seg_offsets", R + 1), ("start_pos", R),
+                 ("total_lens", R), ("want_rows", n_want), ("state_in", R), ("state_out", R)]
+        for g in range(G):
+            sizes.append((f"slots{g}", T))
+            sizes.append((f"bt{g}", R * max_blocks[g]))
+        off = {}
+        total = 0
+        for name, n in sizes:
+            off[name] = (total, n)
+            total += (n + 3) // 4 * 4  # keep every array 16-byte aligned
+        host = self._stage(total)
+        h = host.numpy()
+
+        def seg(name):
+            o, n = off[name]
+            return h[o:o + n]
+
+        seg("token_ids")[:] = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=T)
+        pos = seg("positions")
+        sot = seg("seg_of_token")
+        for i in range(R):
+            a, b = offsets[i], offsets[i + 1]
+            pos[a:b] = np.arange(start[i], start[i] + lens[i])
+            sot[a:b] = i
+        seg("seg_offsets")[:] = offsets
+        seg("start_pos")[:] = start
+        seg("total_lens")[:] = start + lens
+        w = seg("want_rows")
+        k = 0
+        for i, e in enumerate(entries):
+            for x in e.want:
+                w[k] = offsets[i] + x
+                k += 1
+        sin, sout = seg("state_in"), seg("state_out")
+        for i, e in enumerate(entries):
+            sin[i], sout[i] = cache.state_rows(e.req_id)
+        for g in range(G):
+            sl = seg(f"slots{g}")
+            bt = seg(f"bt{g}").reshape(R, max_blocks[g])
+            bt[:] = -1
+            for i, e in enumerate(entries):
+                table = np.asarray(cache.table(e.req_id, g), dtype=np.int64)
+                bt[i, :len(table)] = table
+                p = np.arange(start[i], start[i] + lens[i])
+                pages = table[p // ps]
+                if (pages < 0).any():
+                    raise RuntimeError(f"request {e.req_id!r}: a new token falls on a page already given back")
+                sl[offsets[i]:offsets[i + 1]] = pages * ps + p % ps
+
+        dev = torch.empty((total,), dtype=torch.int32, device=self.device)
+        dev.copy_(host, non_blocking=True)
+        if self.device.type == "cuda":
+            self._copy_done = torch.cuda.Event()
+            self._copy_done.record()
+
+        def dseg(name):
+            o, n = off[name]
+            return dev[o:o + n]
+
+        b = StepBatch()
+        b.T, b.R = T, R
+        b.token_ids, b.positions, b.seg_of_token = dseg("token_ids"), dseg("positions"), dseg("seg_of_token")
+        b.seg_offsets, b.start_pos, b.total_lens = dseg("seg_offsets"), dseg("start_pos"), dseg("total_lens")
+        b.want_rows, b.state_in, b.state_out = dseg("want_rows"), dseg("state_in"), dseg("state_out")
+        b.block_tables = [dseg(f"bt{g}").view(R, max_blocks[g]) for g in range(G)]
+        b.slots = [dseg(f"slots{g}") for g in range(G)]
+        b.num_wanted = n_want
+        b.wants_all_rows = n_want == T and all(list(e.want) == list(range(len(e.tokens))) for e in entries)
+        b.max_q_len = int(lens.max())
+        b.max_total_len = int((start + lens).max())
+        b.max_position = b.max_total_len - 1
+        b.all_decode = bool((lens == 1).all())
+        b.h_seg_offsets = offsets
+        b.h_start_pos = start
+        return b
+
+    # ---- the step -----------------------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry], taps: Optional[dict] = None) -> torch.Tensor:
+        """Runs the entries' tokens as one batch and returns float32 logits [wanted, vocab] in the
+        order of the entries and of each entry's `want`."""
+        batch = self.build_batch(entries)
+        batch.taps = taps
+        logits = self.model.forward(batch, self.cache)
+        for e in entries:
+            self.cache.commit(e.req_id, len(e.tokens))
+        self.steps += 1
+        self.tokens += batch.T
+        return logits

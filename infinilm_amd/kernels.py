@@ -1,0 +1,212 @@
+"""Typed Python faces of the HIP kernels.
+
+Each function checks what the kernel assumes about its operands (device, dtype, contiguity,
+shapes) on the host before the launch, and raises `KernelError` with the kernel's own message
+when it refuses a size.  Nothing here computes on the CPU or through a tensor library: a missing
+library or a CPU tensor is an error.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .csrc import lib as _libmod
+
+F32 = torch.float32
+BF16 = torch.bfloat16
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _lib():
+    return _libmod.load()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {t.dtype}; the kernels take float32 and bfloat16") from None
+
+
+def _dev(*ts: Optional[torch.Tensor]) -> None:
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise KernelError("the kernels run on the GPU only; got a CPU tensor")
+
+
+def _run(name: str, *args) -> None:
+    rc = getattr(_lib(), name)(*args)
+    if rc != 0:
+        raise KernelError(_libmod.last_error())
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _i32(t: torch.Tensor, name: str) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelError(f"{name} must be a contiguous int32 tensor, got {t.dtype}")
+
+
+# ------------------------------------------------------------------------------------------------
+def embed(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+    """float32 residual rows scale * table[ids]."""
+    _dev(ids, table)
+    _i32(ids, "ids")
+    V, H = table.shape
+    if not table.is_contiguous():
+        raise KernelError("embedding table must be contiguous")
+    T = ids.numel()
+    out = torch.empty((T, H), dtype=F32, device=table.device)
+    _run("ilm_embed", out.data_ptr(), ids.data_ptr(), table.data_ptr(), T, H, V, float(scale), _dt(table), _stream())
+    return out
+
+
+def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: torch.Tensor,
+                alpha: float, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """residual += alpha * branch (in place, float32), then its RMS norm times weight, as out_dtype."""
+    _dev(residual, branch, weight)
+    rows, H = residual.shape
+    if residual.dtype != F32 or not residual.is_contiguous():
+        raise KernelError("the residual stream is a contiguous float32 tensor")
+    if branch is not None and (branch.shape != residual.shape or branch.dtype != out_dtype or not branch.is_contiguous()):
+        raise KernelError(f"branch {tuple(branch.shape)} {branch.dtype} does not match residual {tuple(residual.shape)} / {out_dtype}")
+    if weight.shape != (H,) or not weight.is_contiguous():
+        raise KernelError(f"norm weight has shape {tuple(weight.shape)}, expected ({H},)")
+    out = torch.empty((rows, H), dtype=out_dtype, device=residual.device)
+    _run("ilm_add_rmsnorm", out.data_ptr(), residual.data_ptr(), _ptr(branch), weight.data_ptr(), rows, H,
+         float(alpha), float(eps), _DT[out_dtype], _dt(weight), _stream())
+    return out
+
+
+def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                 k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                 slots: Optional[torch.Tensor], nh: int, nkv: int, d: int, rd: int) -> None:
+    """Rotates q and k inside the fused projection rows [T, (nh + 2 nkv) d] and writes k, v to the
+    paged cache [pages, nkv, page, d] at `slots` (None: no write)."""
+    _dev(qkv, positions, cos, sin, k_cache, v_cache, slots)
+    _i32(positions, "positions")
+    T = qkv.shape[0]
+    if qkv.stride(1) != 1 or positions.numel() != T:
+        raise KernelError("qkv rows must be dense and positions must have one entry a token")
+    if cos.dtype != F32 or sin.dtype != F32 or cos.shape != sin.shape or (rd > 0 and cos.shape[1] != rd // 2):
+        raise KernelError(f"rotation tables must be float32 [positions, {rd // 2}], got {tuple(cos.shape)}")
+    page = 0
+    if slots is not None:
+        _i32(slots, "slots")
+        if k_cache is None or v_cache is None or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
+            raise KernelError("cache tensors missing or of another dtype than the activations")
+        if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != d or k_cache.shape != v_cache.shape \
+                or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+            raise KernelError(f"cache shape {tuple(k_cache.shape)} is not [pages, {nkv}, page, {d}]")
+        page = k_cache.shape[2]
+    _run("ilm_rope_kvwrite", qkv.data_ptr(), positions.data_ptr(), cos.data_ptr(), sin.data_ptr(), _ptr(k_cache),
+         _ptr(v_cache), _ptr(slots), T, nh, nkv, d, rd, qkv.stride(0), page, _dt(qkv), _stream())
+
+
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up from rows [gate | up]."""
+    _dev(gate_up)
+    T, two_i = gate_up.shape
+    if two_i % 2 or gate_up.stride(1) != 1:
+        raise KernelError("swiglu takes dense rows of even length")
+    out = torch.empty((T, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _run("ilm_swiglu", out.data_ptr(), gate_up.data_ptr(), T, two_i // 2, gate_up.stride(0), _dt(gate_up), _stream())
+    return out
+
+
+def gather_rows(x: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+    _dev(x, idx)
+    _i32(idx, "row indices")
+    if x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("gather_rows takes a contiguous matrix")
+    out = torch.empty((idx.numel(), x.shape[1]), dtype=x.dtype, device=x.device)
+    _run("ilm_gather_rows", out.data_ptr(), x.data_ptr(), idx.data_ptr(), idx.numel(), x.shape[1], _dt(x), _stream())
+    return out
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, alpha: float = 1.0,
+         out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """alpha * (a w^T + bias); a [M, K] with dense rows, w [N, K]; float accumulation."""
+    _dev(a, w, bias, out)
+    if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
+        raise KernelError(f"gemm shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
+    if a.dtype != w.dtype or a.stride(1) != 1 or w.stride(1) != 1:
+        raise KernelError("gemm operands must share a dtype and have dense rows")
+    M, K = a.shape
+    N = w.shape[0]
+    out_dtype = out_dtype or a.dtype
+    if bias is not None and (bias.shape != (N,) or bias.dtype != w.dtype or not bias.is_contiguous()):
+        raise KernelError(f"bias shape {tuple(bias.shape)} does not fit {N} outputs")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    elif out.shape != (M, N) or out.dtype != out_dtype or out.stride(1) != 1:
+        raise KernelError("gemm output does not fit")
+    _run("ilm_gemm_basic", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0), w.stride(0),
+         out.stride(0), float(alpha), _dt(a), _DT[out_dtype], _stream())
+    return out
+
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                    seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int,
+                    scale: float, window: int = 0) -> torch.Tensor:
+    """Attention of every token over its request's cached keys up to its own position.
+
+    q: rows of T tokens in which head h lies at [h*d, (h+1)*d) (a view into the fused projection is
+    fine); caches [pages, nkv, page, d]; block_tables [R, max_blocks]; returns [T, nh*d]."""
+    _dev(q, k_cache, v_cache, block_tables, seg_of_token, positions)
+    _i32(block_tables, "block_tables")
+    _i32(seg_of_token, "seg_of_token")
+    _i32(positions, "positions")
+    T = q.shape[0]
+    if q.stride(1) != 1 or q.shape[1] < nh * d:
+        raise KernelError("q rows must be dense and hold all query heads")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype or k_cache.shape != v_cache.shape or k_cache.dim() != 4 \
+            or k_cache.shape[1] != nkv or k_cache.shape[3] != d or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError(f"cache {tuple(k_cache.shape)} {k_cache.dtype} is not [pages, {nkv}, page, {d}] of {q.dtype}")
+    if seg_of_token.numel() != T or positions.numel() != T or block_tables.dim() != 2:
+        raise KernelError("per-token metadata does not match the number of tokens")
+    out = torch.empty((T, nh * d), dtype=q.dtype, device=q.device)
+    _run("ilm_attn_basic", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
+         seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d, k_cache.shape[2], block_tables.shape[1],
+         q.stride(0), out.stride(0), float(scale), int(window), _dt(q), _stream())
+    return out
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    _dev(logits)
+    if logits.dtype != F32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("argmax takes float32 rows")
+    n, V = logits.shape
+    out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    _run("ilm_argmax", out.data_ptr(), logits.data_ptr(), n, V, logits.stride(0), _stream())
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           uniform: torch.Tensor) -> torch.Tensor:
+    """One token a row; per-row temperature (float32), top_k (int32), top_p (float32), u in [0,1)."""
+    _dev(logits, temperature, top_k, top_p, uniform)
+    if logits.dtype != F32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("sample takes float32 rows")
+    n, V = logits.shape
+    _i32(top_k, "top_k")
+    for t, nm in ((temperature, "temperature"), (top_p, "top_p"), (uniform, "uniform")):
+        if t.dtype != F32 or t.numel() != n or not t.is_contiguous():
+            raise KernelError(f"{nm} must be float32 with one entry a row")
+    if top_k.numel() != n:
+        raise KernelError("top_k must have one entry a row")
+    out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    _run("ilm_sample", out.data_ptr(), logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
+         uniform.data_ptr(), n, V, logits.stride(0), _stream())
+    return out

@@ -1,0 +1,87 @@
+"""Interfaces of the parts a layer is put together from.
+
+A part is built from its `PartSpec.params` (sizes and constants) and a `BuildContext` (dtype and
+device); it owns its tensors and says under which names they lie in a checkpoint.  No part knows
+which model it is in.
+
+  Norm             forward(stream)                 folds the pending branch into the residual
+                                                   stream and returns the normed activations
+  Mixer            cache_need() -> PagedKV | FixedState | None
+                   forward(x, batch, cache_view)   x [T, hidden] -> [T, hidden]; reads what it
+                                                   needs of the batch (segments, positions) and
+                                                   of its cache view
+  FeedForward      forward(x, batch)               x [T, hidden] -> [T, hidden]
+  PositionEncoding tables()/apply(x, positions)    consumed by mixers
+  Arrangement      forward(stream, batch, cache_view)  wires the slots around the residual stream
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, Optional
+
+import torch
+
+
+@dataclass
+class BuildContext:
+    dtype: torch.dtype
+    device: torch.device
+
+
+class Param:
+    """A named tensor of a part.  `tensor` is where the loader copies to (it may be a view into a
+    fused buffer).  `keep_f32`: a tensor stored in 32-bit in the checkpoint stays 32-bit even when
+    the model runs in bfloat16 (the part's kernels take both)."""
+
+    def __init__(self, tensor: torch.Tensor, keep_f32: bool = False,
+                 replace: Optional[Callable[[torch.Tensor], None]] = None):
+        self.tensor = tensor
+        self.keep_f32 = keep_f32 and replace is not None
+        self._replace = replace
+
+    def replace(self, t: torch.Tensor) -> None:
+        self._replace(t)
+        self.tensor = t
+
+
+class Part:
+    def named_parameters(self) -> Dict[str, Param]:
+        return {}
+
+
+class ResidualStream:
+    """The residual stream in float32 and the branch output that is still to be added to it.
+    The sum `residual += scale * pending` happens inside the next norm's kernel."""
+
+    def __init__(self, residual: torch.Tensor):
+        self.residual = residual
+        self.pending: Optional[torch.Tensor] = None
+        self.pending_scale: float = 1.0
+
+    def push(self, branch: torch.Tensor, scale: float) -> None:
+        if self.pending is not None:
+            raise RuntimeError("a branch is already pending; a norm must fold it first")
+        self.pending = branch
+        self.pending_scale = scale
+
+
+class Norm(Part):
+    def forward(self, stream: ResidualStream) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self):
+        return None
+
+    def forward(self, x: torch.Tensor, batch, cache_view) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    pass

@@ -1,0 +1,46 @@
+"""Dense projections y = alpha * (x W^T + b), W [out, in].
+
+Reference: csrc/layers/linear/base_linear.{hpp,cpp} (alpha, weight layout) and fused_linear.cpp
+(:62-71 the q|k|v split, :90-111 and :163-185 the named row-slices of one fused weight): several
+checkpoint tensors are row ranges of one allocation, so loading by name fills the fused weight and
+one product computes all of them.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .. import kernels
+from .base import BuildContext, Param
+
+
+class FusedLinear:
+    """`out_sizes[i]` rows of the weight belong to the checkpoint tensor `names[i]`."""
+
+    def __init__(self, in_features: int, out_sizes: Sequence[int], names: Sequence[str], bias: bool,
+                 ctx: BuildContext):
+        self.in_features = int(in_features)
+        self.out_sizes = [int(s) for s in out_sizes]
+        self.names = list(names)
+        n = sum(self.out_sizes)
+        self.weight = torch.empty((n, self.in_features), dtype=ctx.dtype, device=ctx.device)
+        self.bias = torch.empty((n,), dtype=ctx.dtype, device=ctx.device) if bias else None
+
+    def named_parameters(self) -> Dict[str, Param]:
+        out: Dict[str, Param] = {}
+        row = 0
+        for name, size in zip(self.names, self.out_sizes):
+            out[f"{name}.weight"] = Param(self.weight[row:row + size])
+            if self.bias is not None:
+                out[f"{name}.bias"] = Param(self.bias[row:row + size])
+            row += size
+        return out
+
+    def forward(self, x: torch.Tensor, alpha: float = 1.0, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return kernels.gemm(x, self.weight, self.bias, alpha, out_dtype)
+
+
+class Linear(FusedLinear):
+    def __init__(self, in_features: int, out_features: int, name: str, bias: bool, ctx: BuildContext):
+        super().__init__(in_features, [out_features], [name], bias, ctx)

@@ -1,0 +1,31 @@
+"""SwiGLU feed-forward: down(silu(gate x) * up x).
+
+Reference: csrc/layers/mlp/mlp.cpp:7-38; gate and up are the two halves (gate first) of one fused
+projection: csrc/layers/linear/fused_linear.cpp:152-158,177-180.
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .. import kernels
+from .base import BuildContext, FeedForward, Param
+from .linear import FusedLinear, Linear
+from .registry import register_feed_forward
+
+
+@register_feed_forward("swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int, bias: bool, ctx: BuildContext):
+        self.gate_up = FusedLinear(hidden_size, [intermediate_size, intermediate_size], ["gate_proj", "up_proj"],
+                                   bias, ctx)
+        self.down = Linear(intermediate_size, hidden_size, "down_proj", bias, ctx)
+
+    def named_parameters(self) -> Dict[str, Param]:
+        out = dict(self.gate_up.named_parameters())
+        out.update(self.down.named_parameters())
+        return out
+
+    def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
+        return self.down.forward(kernels.swiglu(self.gate_up.forward(x)))

@@ -1,0 +1,100 @@
+"""Rotary position encoding with its scaling kinds.
+
+Reference: csrc/layers/rotary_embedding/rotary_embedding.cpp:90-113 (one table for
+max_position_embeddings positions, shared by the layers), rotary_embedding_factory.cpp:11-39 (kind
+from `type` or `rope_type`; absent/null = none), rope_scaling_creators.cpp:23-47,106-115 (longrope's
+keys; `default`, `none`, `dynamic` = no scaling), csrc/config/model_config.hpp:139 (rotate-half
+pairing).  The arithmetic is the tensor library's in the reference; the definition used:
+
+  inv_freq_i = 1 / (f_i * theta^(2i/rd)),  i < rd/2
+  longrope: f = long_factor if max_positions > original_max else short_factor (the table is built
+            once, before any request, so the choice cannot depend on a request's length);
+            s = factor if given and != 1 else max_positions/original_max;
+            m = sqrt(1 + ln s / ln original_max) if s > 1 else 1
+  cos = m cos(p inv_freq), sin = m sin(p inv_freq), angles in float64, tables stored in float32.
+"""
+from __future__ import annotations
+
+import math
+from typing import Callable, Dict, Optional, Tuple
+
+import torch
+
+from .base import BuildContext, PositionEncoding
+from .registry import register_position_encoding
+
+# kind -> function(inv_freq float64 [rd/2], params, max_positions) -> (inv_freq, magnitude)
+SCALINGS: Dict[str, Callable] = {}
+
+
+def register_rope_scaling(kind: str):
+    def deco(fn):
+        SCALINGS[kind] = fn
+        return fn
+    return deco
+
+
+@register_rope_scaling("default")
+@register_rope_scaling("none")
+@register_rope_scaling("dynamic")
+def _no_scaling(inv_freq, params, max_positions):
+    return inv_freq, 1.0
+
+
+@register_rope_scaling("longrope")
+def _longrope(inv_freq, params, max_positions):
+    orig = int(params["original_max_position_embeddings"])
+    factors = params["long_factor"] if max_positions > orig else params["short_factor"]
+    f = torch.tensor(factors, dtype=torch.float64)
+    if f.numel() != inv_freq.numel():
+        raise ValueError(f"longrope factors have {f.numel()} entries, the rotary dimension needs {inv_freq.numel()}")
+    s = float(params.get("factor", 1.0) or 1.0)
+    if s == 1.0:
+        s = max_positions / orig
+    m = math.sqrt(1.0 + math.log(s) / math.log(orig)) if s > 1.0 else 1.0
+    return inv_freq / f, m
+
+
+_TABLE_CACHE: Dict[Tuple, Tuple[torch.Tensor, torch.Tensor]] = {}
+
+
+@register_position_encoding("rotary")
+class RotaryEmbedding(PositionEncoding):
+    """Tables cos/sin [max_positions, rotary_dim/2] float32; layers with equal parameters share them."""
+
+    def __init__(self, head_dim: int, rotary_dim: int, max_positions: int, theta: float,
+                 scaling: Optional[dict], ctx: BuildContext):
+        if rotary_dim % 2 or rotary_dim > head_dim or rotary_dim < 0:
+            raise ValueError(f"rotary_dim {rotary_dim} must be even and at most head_dim {head_dim}")
+        self.head_dim, self.rotary_dim, self.max_positions = int(head_dim), int(rotary_dim), int(max_positions)
+        self.theta = float(theta)
+        self.scaling = scaling
+        key = (self.rotary_dim, self.max_positions, self.theta, repr(scaling), str(ctx.device))
+        if key not in _TABLE_CACHE:
+            cos, sin = self._build()
+            _TABLE_CACHE[key] = (cos.to(ctx.device), sin.to(ctx.device))
+        self.cos, self.sin = _TABLE_CACHE[key]
+
+    def _build(self):
+        rd = self.rotary_dim
+        i = torch.arange(rd // 2, dtype=torch.float64)
+        inv_freq = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float64), 2.0 * i / max(rd, 1))
+        m = 1.0
+        if self.scaling is not None:
+            kind = self.scaling.get("type", self.scaling.get("rope_type"))
+            if kind not in SCALINGS:
+                raise ValueError(f"Unsupported rope_scaling_type: {kind}")
+            inv_freq, m = SCALINGS[kind](inv_freq, self.scaling, self.max_positions)
+        p = torch.arange(self.max_positions, dtype=torch.float64)
+        ang = p[:, None] * inv_freq[None, :]
+        return (torch.cos(ang) * m).to(torch.float32).contiguous(), (torch.sin(ang) * m).to(torch.float32).contiguous()
+
+
+@register_position_encoding("none")
+class NoPositionEncoding(PositionEncoding):
+    """No rotation (rotary_dim 0)."""
+
+    def __init__(self, ctx: BuildContext, head_dim: int = 0, **_):
+        self.head_dim, self.rotary_dim, self.max_positions = int(head_dim), 0, 1 << 30
+        self.cos = torch.zeros((1, 0), dtype=torch.float32, device=ctx.device)
+        self.sin = torch.zeros((1, 0), dtype=torch.float32, device=ctx.device)

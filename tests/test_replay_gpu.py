@@ -1,0 +1,128 @@
+"""The engine against the plain implementation, through the engine's own step function: each
+request alone and whole; most of it in one step and the last 32 tokens one by one; in portions of
+changing size down to two tokens; and mixed, up to four live requests with so few pages that they
+are used again.  In 32-bit and in bfloat16, on tiny configurations that differ in every size."""
+import random
+
+import pytest
+import torch
+
+import plain_minicpm4 as P
+from helpers import CONFIGS, TOL, Driver, make_model_dir, random_tokens, rel_err
+
+pytestmark = pytest.mark.gpu
+
+CASES = [("A", "float32"), ("B", "float32"), ("C", "float32"), ("A", "bfloat16"), ("B", "bfloat16"), ("C", "bfloat16")]
+
+
+@pytest.fixture(scope="module", params=CASES, ids=[f"{c}-{d}" for c, d in CASES])
+def case(request, tmp_path_factory):
+    name, dtype = request.param
+    cfg = CONFIGS[name]()
+    d = tmp_path_factory.mktemp(f"model_{name}_{dtype}")
+    W = make_model_dir(str(d), cfg, seed=100 + ord(name), store=dtype)
+    n_max = min(cfg["max_position_embeddings"], 120)
+    toks = {r: random_tokens(cfg, n, 7 * i + 1) for i, (r, n) in
+            enumerate([("r0", n_max), ("r1", 1), ("r2", 45), ("r3", 70), ("r4", 2), ("r5", 97)])}
+    oracle = {r: P.plain_forward(cfg, W, t) for r, t in toks.items()}
+    return {"cfg": cfg, "dir": str(d), "dtype": dtype, "toks": toks, "oracle": oracle, "name": name}
+
+
+def _check(case, drv, rid):
+    n = len(case["toks"][rid])
+    err = rel_err(drv.request_logits(rid, n), case["oracle"][rid])
+    print(f"[err] {case['name']} {case['dtype']} {rid} n={n}: {err:.3e}")
+    assert err < TOL[case["dtype"]], f"{case['name']} {case['dtype']} request {rid}: error {err:.3e}"
+    return err
+
+
+def test_each_request_alone_and_whole(case):
+    drv = Driver(case["dir"], case["dtype"], num_pages=64, page_size=16)
+    for rid, toks in case["toks"].items():
+        drv.step([(rid, toks)], end=[rid])
+        _check(case, drv, rid)
+    assert drv.runner.cache.free_pages() == 64
+
+
+def test_bulk_then_last_32_one_by_one(case):
+    drv = Driver(case["dir"], case["dtype"], num_pages=16, page_size=8)
+    for rid in ("r0", "r3", "r5"):
+        toks = case["toks"][rid]
+        n = len(toks)
+        drv.step([(rid, toks[:n - 32])])
+        for i in range(n - 32, n):
+            drv.step([(rid, toks[i:i + 1])])
+        _check(case, drv, rid)
+        drv.runner.cache.release(rid)
+
+
+def test_portions_of_changing_size(case):
+    drv = Driver(case["dir"], case["dtype"], num_pages=32, page_size=4)
+    rng = random.Random(5)
+    for rid in ("r0", "r2", "r3", "r5"):
+        toks = case["toks"][rid]
+        i = 0
+        sizes = []
+        forced = [17, 2, 5, 2]
+        while i < len(toks):
+            k = forced.pop(0) if forced else rng.choice([2, 2, 3, 5, 7, 17, 31, 4, 1])
+            k = min(k, len(toks) - i)
+            drv.step([(rid, toks[i:i + k])])
+            sizes.append(k)
+            i += k
+        assert 2 in sizes
+        _check(case, drv, rid)
+        drv.runner.cache.release(rid)
+
+
+def test_mixed_batches_with_page_reuse(case):
+    """Up to four live requests; portions of some beside decoded tokens of others; the pool is so
+    small that pages of finished requests are handed to new ones within the run."""
+    page = 8
+    toks = case["toks"]
+    order = ["r0", "r2", "r1", "r3", "r4", "r5", "r2b", "r0b"]
+    toks = dict(toks, r2b=toks["r2"], r0b=toks["r0"])
+    oracle = dict(case["oracle"], r2b=case["oracle"]["r2"], r0b=case["oracle"]["r0"])
+    need = lambda n: -(-n // page)
+    # pool: enough for the four largest to be live together, far less than the sum of all
+    num_pages = sum(sorted((need(len(t)) for t in toks.values()), reverse=True)[:4])
+    assert num_pages < sum(need(len(t)) for t in toks.values())
+    drv = Driver(case["dir"], case["dtype"], num_pages=num_pages, page_size=page)
+    rng = random.Random(11)
+    waiting = list(order)
+    live = {}          # rid -> tokens fed so far
+    decode_from = {}   # rid -> position from which the request is fed one token a step
+    used_pages = set()
+    while waiting or live:
+        while waiting and len(live) < 4:
+            rid = waiting[0]
+            held = sum(need(len(toks[r])) for r in live)
+            if held + need(len(toks[rid])) > num_pages:
+                break
+            waiting.pop(0)
+            live[rid] = 0
+            decode_from[rid] = max(1, len(toks[rid]) - rng.choice([0, 5, 20]))
+        entries, ending = [], []
+        for rid in list(live):
+            if rng.random() < 0.2 and len(live) > 1:
+                continue  # left out of this step; goes on later
+            done, n = live[rid], len(toks[rid])
+            k = 1 if done >= decode_from[rid] else min(rng.choice([2, 3, 9, 16, 30]), decode_from[rid] - done)
+            entries.append((rid, toks[rid][done:done + k]))
+            live[rid] = done + k
+            if live[rid] == n:
+                ending.append(rid)
+        if not entries:
+            continue
+        drv.step(entries, end=ending)
+        for rid, _ in entries:
+            if rid not in ending:
+                used_pages.update(drv.runner.cache.table(rid, 0))
+        for rid in ending:
+            del live[rid]
+    for rid in order:
+        err = rel_err(drv.request_logits(rid, len(toks[rid])), oracle[rid])
+        print(f"[err] mixed {case['name']} {case['dtype']} {rid}: {err:.3e}")
+        assert err < TOL[case["dtype"]], f"{case['name']} {case['dtype']} request {rid}: error {err:.3e}"
+    assert drv.runner.cache.free_pages() == num_pages
+    drv.runner.cache.check()
