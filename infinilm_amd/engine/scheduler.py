@@ -1,0 +1,273 @@
+"""The scheduler: admits requests, cuts prompts into portions under a token budget, decodes,
+finishes and frees, and decides what happens when pages run out.
+
+Reference: python/infinilm/llm/scheduler.py: FIFO waiting and running queues (:75-76), admission
+with a token budget (:111-127) and a worst-case page check (:453-495), head-of-line blocking
+(:202-215), a step is either all prompts or all decodes (:295-366), finishing frees pages
+(:404-451).  The reference never cuts a prompt and never preempts: running out of pages in a
+decode raises (python/infinilm/llm/cache_manager.py:321-324).
+
+Here every step holds the running requests' decode tokens first, then portions of prompts (those
+already begun, then new admissions) until the token budget or the batch size is used up.  Two
+admission policies:
+  reserve_full  the reference's check: a request enters only if the pages for its prompt and
+                its max_tokens, plus what every running request may still need, fit the pool;
+                pages then never run out.
+  optimistic    a request enters if its first portion fits now.  When a later token finds no page,
+                the most recently admitted running request is preempted: its pages go back, it
+                returns to the front of the waiting queue and is recomputed (prompt and generated
+                tokens) when it is admitted again.  A request that cannot fit the pool alone fails
+                with FinishReason.ERROR when it is added.
+The scheduler never touches the GPU: it plans against the cache manager's page counts.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, List, Optional
+
+from ..cache import CacheManager
+from .request import FinishReason, InferenceRequest, RequestStatus
+
+
+@dataclass
+class ScheduledEntry:
+    request: InferenceRequest
+    start: int            # index of the first token of the portion in request.all_token_ids()
+    num_tokens: int
+    samples: bool         # the portion ends at the last known token: a new token is sampled from it
+
+
+@dataclass
+class SchedulerOutput:
+    entries: List[ScheduledEntry] = field(default_factory=list)
+    preempted: List[InferenceRequest] = field(default_factory=list)
+
+    @property
+    def num_tokens(self) -> int:
+        return sum(e.num_tokens for e in self.entries)
+
+
+class Scheduler:
+    def __init__(self, cache: CacheManager, max_num_seqs: int, max_num_batched_tokens: int,
+                 chunk_size: Optional[int] = None, policy: str = "optimistic", max_positions: int = 1 << 30):
+        if policy not in ("optimistic", "reserve_full"):
+            raise ValueError(f"unknown admission policy {policy!r}")
+        if max_num_seqs <= 0 or max_num_batched_tokens <= 0:
+            raise ValueError("max_num_seqs and max_num_batched_tokens must be positive")
+        self.cache = cache
+        self.max_num_seqs = int(max_num_seqs)
+        self.max_num_batched_tokens = int(max_num_batched_tokens)
+        self.chunk_size = int(chunk_size or max_num_batched_tokens)
+        self.policy = policy
+        self.max_positions = int(max_positions)
+        self.waiting: Deque[InferenceRequest] = deque()
+        self.running: List[InferenceRequest] = []
+        self.finished: List[InferenceRequest] = []
+        self._admissions = 0
+        self.num_preemptions = 0
+        self.log: List[Dict] = []  # composition of each step
+
+    # ---- adding ---------------------------------------------------------------------------------
+    def _pages_for(self, n_tokens: int) -> int:
+        return -(-n_tokens // self.cache.page_size)
+
+    def add_request(self, req: InferenceRequest) -> None:
+        n = req.get_prompt_length()
+        if n == 0:
+            self._fail(req, "empty prompt")
+            return
+        if n >= self.max_positions:
+            self._fail(req, f"prompt of {n} tokens leaves no room under max_position_embeddings {self.max_positions}")
+            return
+        smallest_pool = min((g.pool.num_pages for g in self.cache.groups), default=1 << 30)
+        if self._pages_for(n + 1) > smallest_pool:
+            self._fail(req, f"no_capacity: prompt of {n} tokens needs {self._pages_for(n + 1)} pages, the pool has {smallest_pool}")
+            return
+        if self.policy == "reserve_full":
+            worst = self._pages_for(min(n + req.sampling_params.max_tokens, self.max_positions))
+            if worst > smallest_pool:
+                self._fail(req, f"no_capacity: prompt and max_tokens need {worst} pages, the pool has {smallest_pool}")
+                return
+        req.status = RequestStatus.WAITING
+        self.waiting.append(req)
+
+    def _fail(self, req: InferenceRequest, why: str) -> None:
+        req.status = RequestStatus.FAILED
+        req.finish_reason = FinishReason.ERROR
+        req.error = why
+        self.finished.append(req)
+
+    def has_unfinished(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    # ---- planning -------------------------------------------------------------------------------
+    def _fits(self, req: InferenceRequest, n: int, promised: List[int]) -> bool:
+        need = self.cache.pages_needed(req.request_id, n)
+        return all(p + k <= g.pool.num_free for p, k, g in zip(promised, need, self.cache.groups))
+
+    def _promise(self, req: InferenceRequest, n: int, promised: List[int]) -> None:
+        for i, k in enumerate(self.cache.pages_needed(req.request_id, n)):
+            promised[i] += k
+
+    def _worst_case_pages(self, req: InferenceRequest) -> int:
+        """Pages the request may still take: up to prompt + max_tokens (scheduler.py:453-495)."""
+        total = min(req.get_prompt_length() + req.sampling_params.max_tokens, self.max_positions)
+        held = len(self.cache.table(req.request_id, 0)) if self.cache.has(req.request_id) and self.cache.groups else 0
+        return max(0, self._pages_for(total) - held)
+
+    def _can_admit(self, req: InferenceRequest, first_portion: int, promised: List[int]) -> bool:
+        if self.policy == "reserve_full":
+            need = self._pages_for(min(req.get_prompt_length() + req.sampling_params.max_tokens, self.max_positions))
+            need += sum(self._worst_case_pages(r) for r in self.running)
+            return all(need <= g.pool.num_free for g in self.cache.groups)
+        need = self._pages_for(first_portion)
+        return all(p + need <= g.pool.num_free for p, g in zip(promised, self.cache.groups))
+
+    def _preempt(self, victim: InferenceRequest, out: SchedulerOutput) -> None:
+        self.cache.release(victim.request_id)
+        self.running.remove(victim)
+        victim.num_computed_tokens = 0
+        victim.status = RequestStatus.WAITING
+        victim.num_preemptions += 1
+        self.num_preemptions += 1
+        self.waiting.appendleft(victim)
+        out.preempted.append(victim)
+
+    def schedule(self) -> SchedulerOutput:
+        out = SchedulerOutput()
+        promised = [0] * len(self.cache.groups)
+        budget = self.max_num_batched_tokens
+
+        def plan(req: InferenceRequest, n: int) -> None:
+            nonlocal budget
+            start = req.num_computed_tokens
+            self._promise(req, n, promised)
+            out.entries.append(ScheduledEntry(req, start, n, start + n == req.num_known_tokens()))
+            budget -= n
+
+        # 1. decode tokens of running requests, oldest first; make room by preempting the newest
+        for req in sorted(self.running, key=lambda r: r.admission_index):
+            if req not in self.running:       # preempted while serving an older one
+                continue
+            if req.num_known_tokens() - req.num_computed_tokens != 1 or req.get_num_generated_tokens() == 0:
+                continue
+            if budget <= 0:
+                break
+            while not self._fits(req, 1, promised):
+                victim = max(self.running, key=lambda r: r.admission_index)
+                if victim is req and len(self.running) == 1:
+                    # alone with the whole pool and still short of a page: it can never finish
+                    self.cache.release(req.request_id)
+                    self.running.remove(req)
+                    self._fail(req, "no_capacity: the request cannot make progress with the whole pool to itself")
+                    break
+                planned = [e for e in out.entries if e.request is victim]
+                if planned:                   # never happens for decodes planned oldest-first, kept for safety
+                    out.entries.remove(planned[0])
+                self._preempt(victim, out)
+                if victim is req:
+                    break
+            if req in self.running:
+                plan(req, 1)
+        # 2. portions of prompts already begun (and recomputations after a preemption)
+        for req in sorted(self.running, key=lambda r: r.admission_index):
+            left = req.num_known_tokens() - req.num_computed_tokens
+            if any(e.request is req for e in out.entries) or left <= 0 or budget <= 0:
+                continue
+            n = min(left, self.chunk_size, budget)
+            while n > 0 and not self._fits(req, n, promised):
+                # take what the free pages allow; a portion may end anywhere
+                free_tokens = min((g.pool.num_free - p) for g, p in zip(self.cache.groups, promised)) * self.cache.page_size
+                room_in_last_page = (-self.cache.length(req.request_id)) % self.cache.page_size
+                n = min(n - 1, free_tokens + room_in_last_page)
+            if n > 0:
+                plan(req, n)
+        # 3. admissions, first come first served; the first that does not fit blocks the rest
+        while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
+            req = self.waiting[0]
+            if req in out.preempted:          # just made room for an older request: wait a step
+                break
+            n = min(req.num_known_tokens(), self.chunk_size, budget)
+            if not self._can_admit(req, n, promised):
+                break
+            self.waiting.popleft()
+            self.cache.admit(req.request_id)
+            req.status = RequestStatus.RUNNING
+            req.admission_index = self._admissions
+            self._admissions += 1
+            self.running.append(req)
+            plan(req, n)
+        # 4. nothing can move although requests are running: everything waits for pages that only a
+        #    preemption can free
+        if not out.entries and self.running:
+            victim = max(self.running, key=lambda r: r.admission_index)
+            if len(self.running) == 1:
+                self.cache.release(victim.request_id)
+                self.running.remove(victim)
+                self._fail(victim, "no_capacity: the request cannot make progress with the whole pool to itself")
+            else:
+                self._preempt(victim, out)
+                return self._merge(out, self.schedule())
+        self.log.append({"decode": sum(1 for e in out.entries if e.num_tokens == 1 and e.start > 0),
+                         "portions": [e.num_tokens for e in out.entries if not (e.num_tokens == 1 and e.start > 0)],
+                         "preempted": len(out.preempted), "free_pages": [g.pool.num_free for g in self.cache.groups]})
+        return out
+
+    @staticmethod
+    def _merge(first: SchedulerOutput, second: SchedulerOutput) -> SchedulerOutput:
+        second.preempted = first.preempted + second.preempted
+        return second
+
+    # ---- after the step -----------------------------------------------------------------------
+    def update(self, out: SchedulerOutput, sampled: Dict[str, int]) -> List[InferenceRequest]:
+        """Advances the requests by what ran; `sampled[request_id]` is the new token of every entry
+        with `samples`.  Returns the requests that finished in this step (their pages are free)."""
+        done = []
+        for e in out.entries:
+            req = e.request
+            req.num_computed_tokens += e.num_tokens
+            if not e.samples:
+                continue
+            tok = int(sampled[req.request_id])
+            req.output_token_ids.append(tok)
+            reason = self._finish_reason(req, tok)
+            if reason is not None:
+                req.finish_reason = reason
+                req.status = RequestStatus.FINISHED
+                self.cache.release(req.request_id)
+                self.running.remove(req)
+                self.finished.append(req)
+                done.append(req)
+        return done
+
+    def _finish_reason(self, req: InferenceRequest, tok: int) -> Optional[FinishReason]:
+        """python/infinilm/llm/llm.py:279-303, plus stop_token_ids and the position limit."""
+        sp = req.sampling_params
+        if req.get_num_generated_tokens() >= sp.max_tokens:
+            return FinishReason.LENGTH
+        if not sp.ignore_eos:
+            if tok in req.eos_token_ids:
+                return FinishReason.EOS_TOKEN
+            if tok in sp.stop_token_ids:
+                return FinishReason.STOP
+        if req.num_known_tokens() >= self.max_positions:
+            return FinishReason.LENGTH
+        return None
+
+    def abort(self, req: InferenceRequest) -> None:
+        if req in self.running:
+            self.cache.release(req.request_id)
+            self.running.remove(req)
+        elif req in self.waiting:
+            self.waiting.remove(req)
+        else:
+            return
+        req.status = RequestStatus.CANCELED
+        req.finish_reason = FinishReason.CANCELED
+        self.finished.append(req)
+
+    def get_cache_stats(self) -> dict:
+        s = self.cache.stats()
+        s.update({"waiting": len(self.waiting), "running": len(self.running), "preemptions": self.num_preemptions})
+        return s

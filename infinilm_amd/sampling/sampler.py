@@ -1,0 +1,55 @@
+"""From rows of logits to tokens: argmax for greedy rows, temperature / top-k / top-p otherwise.
+
+Reference: one `random_sample_(out, row, random_val, top_p, top_k, temperature)` call per request
+in a host loop, random_val from a `std::mt19937` seeded by `std::random_device`
+(csrc/engine/rank_worker.cpp:27,467-513): not reproducible.  Here all rows are sampled by one
+kernel launch, and the uniform number of a row is a pure function of (seed, request, index of the
+generated token), so a request's tokens do not depend on what else is in the batch or on how often
+it was preempted.
+"""
+from __future__ import annotations
+
+from typing import List, Sequence, Tuple
+
+import torch
+
+from .. import kernels
+from .params import SamplingParams
+
+_MASK = (1 << 64) - 1
+
+
+def _mix(x: int) -> int:
+    """splitmix64 finaliser."""
+    x = (x + 0x9E3779B97F4A7C15) & _MASK
+    x = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    x = ((x ^ (x >> 27)) * 0x94D2049BB133111B) & _MASK
+    return x ^ (x >> 31)
+
+
+def uniform_for(seed: int, request_key: int, index: int) -> float:
+    """u in [0, 1) with 24 bits, a pure function of its arguments."""
+    x = _mix(_mix(_mix(seed & _MASK) ^ (request_key & _MASK)) ^ (index & _MASK))
+    return (x >> 40) / float(1 << 24)
+
+
+class Sampler:
+    def __init__(self, seed: int = 0):
+        self.seed = int(seed)
+
+    def sample(self, logits: torch.Tensor, rows: Sequence[Tuple[SamplingParams, int, int]]) -> List[int]:
+        """`rows[i]` = (params, request key, index of the token being generated) for logits[i]."""
+        n = logits.shape[0]
+        if n != len(rows):
+            raise ValueError(f"{n} rows of logits for {len(rows)} requests")
+        if n == 0:
+            return []
+        if all(p.greedy for p, _, _ in rows):
+            return kernels.argmax(logits).tolist()
+        dev = logits.device
+        temp = torch.tensor([p.temperature for p, _, _ in rows], dtype=torch.float32).to(dev)
+        top_k = torch.tensor([p.top_k for p, _, _ in rows], dtype=torch.int32).to(dev)
+        top_p = torch.tensor([p.top_p for p, _, _ in rows], dtype=torch.float32).to(dev)
+        u = torch.tensor([uniform_for(self.seed if p.seed is None else p.seed, key, idx) for p, key, idx in rows],
+                         dtype=torch.float32).to(dev)
+        return kernels.sample(logits, temp, top_k, top_p, u).tolist()
