@@ -2,7 +2,7 @@
 entries with the same need, and slots of fixed-size state per request.
 
 Reference: data plane csrc/cache/kv_cache.cpp:113-148 (one tensor per layer, here K and V apart,
-each [pages, nkv, page, d]); control plane python/infinilm/llm/cache_manager.py:158-191 (pages for
+keys [pages, nkv, page, d], values [pages, nkv, d, page]); control plane python/infinilm/llm/cache_manager.py:158-191 (pages for
 a prompt), :317-328 (a new page iff the new token opens one), :330-348 (giving back); fixed-size
 state csrc/cache/mamba_cache.cpp:8-47 and cache_manager.py:33-68 (row 0 is the zero state, rows
 from a free list).  Differences by design: pages are reserved portion by portion instead of for
@@ -87,9 +87,13 @@ class CacheManager:
         for e, need in enumerate(self.needs):
             if isinstance(need, PagedKV):
                 n = self.groups[self.group_of_entry[e]].pool.num_pages
-                shape = (n, need.num_kv_heads, self.page_size, need.head_dim)
-                self.k[e] = torch.zeros(shape, dtype=dtype, device=self.device)
-                self.v[e] = torch.zeros(shape, dtype=dtype, device=self.device)
+                # keys [pages, nkv, page, d]; values transposed [pages, nkv, d, page], so that the
+                # attention kernels read consecutive keys of one dim with one load.  Zero-filled once:
+                # what a reused page holds is stale but finite, and lengths bound every read.
+                self.k[e] = torch.zeros((n, need.num_kv_heads, self.page_size, need.head_dim), dtype=dtype,
+                                        device=self.device)
+                self.v[e] = torch.zeros((n, need.num_kv_heads, need.head_dim, self.page_size), dtype=dtype,
+                                        device=self.device)
             elif isinstance(need, FixedState):
                 self.state[e] = torch.zeros((self.max_requests + 1,) + tuple(need.shape),
                                             dtype=need.dtype or torch.float32, device=self.device)

@@ -4,7 +4,7 @@
 // Contract (shared by every attention kernel here): token t belongs to request seg[t] and sits at
 // absolute position pos[t]; it sees the keys of its request at positions [lo, pos[t]] with
 // lo = max(0, pos[t] - window + 1) when window > 0, else 0.  Keys and values are read from the
-// paged cache [pages, nkv, page, d] through block_tables[seg[t], key / page]; the step has
+// paged cache (keys [pages, nkv, page, d], values transposed [pages, nkv, d, page]) through block_tables[seg[t], key / page]; the step has
 // already written this step's keys there.  Keys are consumed in tiles of 64 aligned to absolute
 // key index, so the order of every sum is fixed by (request, position) alone: cutting a prompt
 // into portions or batching it with other requests cannot change a bit of the result.
@@ -54,12 +54,12 @@ attn_basic_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __restr
         for (int j = j0; j <= j1; ++j) {
             const int key = (tile << 6) + j;
             const int pg = bt[key / page];
-            const T* vrow = vc + (((size_t)pg * nkv + kvh) * page + (key % page)) * d;
+            const T* vcol = vc + ((size_t)pg * nkv + kvh) * d * page + (key % page);
             const float w = ps[j];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int dim = lane + 64 * i;
-                if (dim < d) acc[i] = fmaf(w, to_f32(vrow[dim]), acc[i]);
+                if (dim < d) acc[i] = fmaf(w, to_f32(vcol[(size_t)dim * page]), acc[i]);
             }
         }
         __syncthreads();

@@ -89,9 +89,9 @@ extern "C" int ilm_add_rmsnorm(void* x, void* r, const void* h, const void* w, i
 
 // ------------------------------------------------------------------------------------------
 // Rotation of q and k in place (pairs (i, i + rd/2), tables cos/sin [max_pos, rd/2] float), and
-// the write of the rotated k and of v into the paged cache [pages, nkv, page, d] at
-// slot = page_id * page + offset.  One block of 64 threads per (token, head slot); head slots
-// are nh query heads, then nkv key heads, then nkv value heads, as they lie in the qkv row.
+// the write of the rotated k into the paged cache [pages, nkv, page, d] and of v into
+// [pages, nkv, d, page], at slot = page_id * page + offset.  One block of 64 threads per
+// (token, head slot); head slots are nh query heads, then nkv key heads, then nkv value heads, as they lie in the qkv row.
 // slot < 0: nothing is written to the cache for that token.
 // ------------------------------------------------------------------------------------------
 template <typename T>
@@ -106,17 +106,17 @@ rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ pos, const floa
     const bool is_v = hs >= nh + nkv;
     const bool is_k = !is_v && hs >= nh;
     T* dst = nullptr;
-    if ((is_k || is_v) && slots != nullptr) {
+    if (is_k && slots != nullptr) {
         const int slot = slots[t];
-        if (slot >= 0) {
-            const int kvh = is_k ? hs - nh : hs - nh - nkv;
-            const size_t off = (((size_t)(slot / page) * nkv + kvh) * page + (slot % page)) * d;
-            dst = (is_k ? kc : vc) + off;
-        }
+        if (slot >= 0) dst = kc + (((size_t)(slot / page) * nkv + (hs - nh)) * page + (slot % page)) * d;
     }
     if (is_v) {
-        if (dst != nullptr)
-            for (int i = threadIdx.x; i < d; i += 64) dst[i] = p[i];
+        // values are cached transposed, [pages, nkv, d, page]: consecutive keys of one dim are contiguous
+        if (slots != nullptr && slots[t] >= 0) {
+            const int slot = slots[t];
+            T* vdst = vc + ((size_t)(slot / page) * nkv + (hs - nh - nkv)) * d * page + (slot % page);
+            for (int i = threadIdx.x; i < d; i += 64) vdst[(size_t)i * page] = p[i];
+        }
         return;
     }
     const float* c = cosT + (size_t)pos[t] * half;

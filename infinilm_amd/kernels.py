@@ -7,6 +7,7 @@ library or a CPU tensor is an error.
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -16,6 +17,10 @@ from .csrc import lib as _libmod
 F32 = torch.float32
 BF16 = torch.bfloat16
 _DT = {torch.float32: 0, torch.bfloat16: 1}
+ATT_CHUNK = 256  # keys per chunk of the matrix-core attention kernel (ilm_attn_mfma_chunk())
+# INFINILM_AMD_BASIC=1 runs the plain kernels everywhere (for telling a kernel's fault from the engine's)
+FORCE_BASIC = os.environ.get("INFINILM_AMD_BASIC", "0") == "1"
+USE_LIBRARY_GEMM = os.environ.get("INFINILM_AMD_LIBRARY_GEMM", "1") == "1"
 
 
 class KernelError(RuntimeError):
@@ -51,6 +56,16 @@ def _run(name: str, *args) -> None:
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
+
+
+def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int) -> int:
+    """Keys [pages, nkv, page, d], values transposed [pages, nkv, d, page]; returns the page size."""
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != d \
+            or tuple(v_cache.shape) != (k_cache.shape[0], nkv, d, k_cache.shape[2]) \
+            or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise KernelError(f"cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)} are not "
+                          f"[pages, {nkv}, page, {d}] / [pages, {nkv}, {d}, page]")
+    return k_cache.shape[2]
 
 
 def _i32(t: torch.Tensor, name: str) -> None:
@@ -106,10 +121,7 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, 
         _i32(slots, "slots")
         if k_cache is None or v_cache is None or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
             raise KernelError("cache tensors missing or of another dtype than the activations")
-        if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != d or k_cache.shape != v_cache.shape \
-                or not k_cache.is_contiguous() or not v_cache.is_contiguous():
-            raise KernelError(f"cache shape {tuple(k_cache.shape)} is not [pages, {nkv}, page, {d}]")
-        page = k_cache.shape[2]
+        page = _check_cache(k_cache, v_cache, nkv, d)
     _run("ilm_rope_kvwrite", qkv.data_ptr(), positions.data_ptr(), cos.data_ptr(), sin.data_ptr(), _ptr(k_cache),
          _ptr(v_cache), _ptr(slots), T, nh, nkv, d, rd, qkv.stride(0), page, _dt(qkv), _stream())
 
@@ -152,6 +164,18 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     elif out.shape != (M, N) or out.dtype != out_dtype or out.stride(1) != 1:
         raise KernelError("gemm output does not fit")
+    if a.dtype == BF16 and not FORCE_BASIC:
+        aligned = K % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 \
+            and w.data_ptr() % 16 == 0
+        if M <= 64 and aligned:
+            _run("ilm_gemm_skinny", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
+                 w.stride(0), out.stride(0), float(alpha), _DT[out_dtype], _stream())
+            return out
+        if M > 64 and bias is None and alpha == 1.0 and out_dtype == BF16 and USE_LIBRARY_GEMM:
+            # large products go to the vendor library, as the reference's linear layers do
+            # (csrc/layers/quantization/none_quantization.cpp:26-46 calls its library's linear)
+            torch.matmul(a, w.t(), out=out)
+            return out
     _run("ilm_gemm_basic", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0), w.stride(0),
          out.stride(0), float(alpha), _dt(a), _DT[out_dtype], _stream())
     return out
@@ -159,11 +183,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int,
-                    scale: float, window: int = 0) -> torch.Tensor:
+                    scale: float, window: int = 0, max_total_len: Optional[int] = None) -> torch.Tensor:
     """Attention of every token over its request's cached keys up to its own position.
 
     q: rows of T tokens in which head h lies at [h*d, (h+1)*d) (a view into the fused projection is
-    fine); caches [pages, nkv, page, d]; block_tables [R, max_blocks]; returns [T, nh*d]."""
+    fine); caches as the cache manager lays them out; block_tables [R, max_blocks]; `max_total_len`: an
+    upper bound of position + 1 over the batch (the matrix-core kernel sizes its key chunks by it;
+    without it the plain kernel runs).  Returns [T, nh*d]."""
     _dev(q, k_cache, v_cache, block_tables, seg_of_token, positions)
     _i32(block_tables, "block_tables")
     _i32(seg_of_token, "seg_of_token")
@@ -171,14 +197,25 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     T = q.shape[0]
     if q.stride(1) != 1 or q.shape[1] < nh * d:
         raise KernelError("q rows must be dense and hold all query heads")
-    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype or k_cache.shape != v_cache.shape or k_cache.dim() != 4 \
-            or k_cache.shape[1] != nkv or k_cache.shape[3] != d or not k_cache.is_contiguous() or not v_cache.is_contiguous():
-        raise KernelError(f"cache {tuple(k_cache.shape)} {k_cache.dtype} is not [pages, {nkv}, page, {d}] of {q.dtype}")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise KernelError(f"cache dtype {k_cache.dtype} differs from the activations' {q.dtype}")
+    page = _check_cache(k_cache, v_cache, nkv, d)
     if seg_of_token.numel() != T or positions.numel() != T or block_tables.dim() != 2:
         raise KernelError("per-token metadata does not match the number of tokens")
     out = torch.empty((T, nh * d), dtype=q.dtype, device=q.device)
+    if (q.dtype == BF16 and not FORCE_BASIC and d % 16 == 0 and d <= 128 and page % 16 == 0 and q.stride(0) % 8 == 0
+            and max_total_len is not None):
+        nsplit = max(1, -(-int(max_total_len) // ATT_CHUNK))
+        ws_acc = ws_ml = None
+        if nsplit > 1:
+            ws_acc = torch.empty((T * nh * nsplit * d,), dtype=F32, device=q.device)
+            ws_ml = torch.empty((T * nh * nsplit * 2,), dtype=F32, device=q.device)
+        _run("ilm_attn_mfma", out.data_ptr(), _ptr(ws_acc), _ptr(ws_ml), q.data_ptr(), k_cache.data_ptr(),
+             v_cache.data_ptr(), block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d,
+             page, block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window), nsplit, _stream())
+        return out
     _run("ilm_attn_basic", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
-         seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d, k_cache.shape[2], block_tables.shape[1],
+         seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d, page, block_tables.shape[1],
          q.stride(0), out.stride(0), float(scale), int(window), _dt(q), _stream())
     return out
 

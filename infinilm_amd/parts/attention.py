@@ -53,5 +53,6 @@ class GQAttention(Mixer):
         if batch.taps is not None:
             batch.taps.setdefault("qkv_rotated", []).append(qkv.clone())
         o = kernels.paged_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,
-                                    batch.positions, self.nh, self.nkv, self.d, self.scale, self.window)
+                                    batch.positions, self.nh, self.nkv, self.d, self.scale, self.window,
+                                    batch.max_total_len)
         return self.o_proj.forward(o)

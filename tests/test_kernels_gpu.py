@@ -1,0 +1,272 @@
+"""Each HIP kernel alone against a plain PyTorch float64 reference of the same op, at other sizes
+than the engine tests use: odd widths, head sizes in steps of 16, groups of 1 to 16 heads, contexts
+that cross pages and key chunks, a far key that must dominate, a window's edge."""
+import math
+
+import pytest
+import torch
+
+import plain_minicpm4 as P
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+F64 = torch.float64
+
+
+@pytest.fixture(scope="module")
+def K():
+    from infinilm_amd import kernels
+    return kernels
+
+
+def _rand(shape, seed, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def _close(got, want, tol):
+    got = got.detach().cpu().to(F64)
+    want = want.detach().cpu().to(F64)
+    err = float((got - want).abs().max() / max(1.0, float(want.abs().max())))
+    assert err < tol, f"error {err:.3e} above {tol:.1e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(K, dtype):
+    table = _rand((331, 80), 1, dtype)
+    ids = torch.tensor([0, 330, 7, 7, 100], dtype=torch.int32)
+    out = K.embed(ids.to(DEV), table.to(DEV), 7.5)
+    assert out.dtype == torch.float32
+    _close(out, table.to(F64)[ids.long()] * 7.5, 1e-6)
+
+
+@pytest.mark.parametrize("dtype,wdtype,H", [(torch.float32, torch.float32, 80), (torch.bfloat16, torch.bfloat16, 331),
+                                            (torch.bfloat16, torch.float32, 4096), (torch.float32, torch.float32, 1)])
+def test_add_rmsnorm(K, dtype, wdtype, H):
+    r = _rand((5, H), 2, scale=3.0)
+    h = _rand((5, H), 3, dtype)
+    w = _rand((H,), 4, wdtype) + 1
+    rd = r.to(DEV).clone()
+    x = K.add_rmsnorm(rd, h.to(DEV), w.to(DEV), 0.37, 1e-5, dtype)
+    want_r = r.to(F64) + 0.37 * h.to(F64)
+    _close(rd, want_r, 1e-6)
+    want = P.plain_rmsnorm(want_r, w.to(F64), 1e-5)
+    _close(x, want, 2e-6 if dtype == torch.float32 else 1e-2)
+    # without a branch the residual is untouched
+    rd2 = r.to(DEV).clone()
+    x2 = K.add_rmsnorm(rd2, None, w.to(DEV), 1.0, 1e-5, dtype)
+    assert torch.equal(rd2.cpu(), r)
+    _close(x2, P.plain_rmsnorm(r.to(F64), w.to(F64), 1e-5), 2e-6 if dtype == torch.float32 else 1e-2)
+    # a row's result does not depend on the batch around it
+    x1 = K.add_rmsnorm(r[2:3].to(DEV).clone(), None, w.to(DEV), 1.0, 1e-5, dtype)
+    assert torch.equal(x1.cpu(), x2[2:3].cpu())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,d,rd,page", [(4, 2, 16, 16, 4), (3, 1, 48, 48, 16), (5, 5, 32, 16, 8), (2, 1, 80, 0, 16)])
+def test_rope_and_cache_write(K, dtype, nh, nkv, d, rd, page):
+    T, max_pos = 9, 50
+    qkv = _rand((T, (nh + 2 * nkv) * d), 5, dtype)
+    pos = torch.tensor([0, 1, 2, 17, 49, 3, 3, 30, 11], dtype=torch.int32)
+    cfg = {"hidden_size": d, "num_attention_heads": 1, "max_position_embeddings": max_pos, "rope_theta": 777.0,
+           "partial_rotary_factor": rd / d if 0 < rd < d else 1.0}
+    if rd > 0:
+        cos, sin = P.plain_rope_tables(cfg)
+    else:
+        cos, sin = torch.zeros(max_pos, 0, dtype=F64), torch.zeros(max_pos, 0, dtype=F64)
+    n_pages = 7
+    kc = torch.zeros((n_pages, nkv, page, d), dtype=dtype, device=DEV)
+    vc = torch.zeros((n_pages, nkv, d, page), dtype=dtype, device=DEV)
+    slots = torch.tensor([5 * page + 1, 0, 2 * page + page - 1, -1, 6 * page, 3 * page + 2, page, page + 1, 4 * page],
+                         dtype=torch.int32)
+    buf = qkv.to(DEV).clone()
+    K.rope_kvwrite(buf, pos.to(DEV), cos.float().to(DEV), sin.float().to(DEV), kc, vc, slots.to(DEV), nh, nkv, d, rd)
+    x = qkv.to(F64).view(T, nh + 2 * nkv, d)
+    want_q = P.plain_apply_rope(x[:, :nh], pos, cos, sin, rd) if rd else x[:, :nh]
+    want_k = P.plain_apply_rope(x[:, nh:nh + nkv], pos, cos, sin, rd) if rd else x[:, nh:nh + nkv]
+    tol = 2e-6 if dtype == torch.float32 else 1e-2
+    got = buf.cpu().view(T, nh + 2 * nkv, d)
+    _close(got[:, :nh], want_q, tol)
+    _close(got[:, nh:nh + nkv], want_k, tol)
+    assert torch.equal(got[:, nh + nkv:], qkv.view(T, nh + 2 * nkv, d)[:, nh + nkv:])   # v untouched
+    for t in range(T):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        pg, off = s // page, s % page
+        assert torch.equal(kc[pg, :, off, :].cpu(), got[t, nh:nh + nkv])        # the rotated key is what is cached
+        assert torch.equal(vc[pg, :, :, off].cpu(), got[t, nh + nkv:])           # values lie transposed
+    written = {int(s) for s in slots if s >= 0}
+    mask = torch.ones(n_pages * page, dtype=torch.bool)
+    mask[list(written)] = False
+    assert not kc.cpu().permute(0, 2, 1, 3).reshape(n_pages * page, -1)[mask].any()  # nothing else was touched
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_and_gather(K, dtype):
+    gu = _rand((7, 2 * 200), 6, dtype, 2.0)
+    out = K.swiglu(gu.to(DEV))
+    g, u = gu.to(F64)[:, :200], gu.to(F64)[:, 200:]
+    _close(out, P.plain_swiglu(g, u), 2e-6 if dtype == torch.float32 else 1e-2)
+    x = _rand((11, 96), 7, dtype)
+    idx = torch.tensor([10, 0, 3, 3], dtype=torch.int32)
+    assert torch.equal(K.gather_rows(x.to(DEV), idx.to(DEV)).cpu(), x[idx.long()])
+
+
+@pytest.mark.parametrize("M,N,K_", [(1, 1, 1), (5, 331, 80), (64, 96, 200), (130, 70, 33), (3, 4608, 4096)])
+def test_gemm_float32_is_true_float32(K, M, N, K_):
+    a, w, b = _rand((M, K_), 8), _rand((N, K_), 9), _rand((N,), 10)
+    out = K.gemm(a.to(DEV), w.to(DEV), b.to(DEV), 0.25)
+    want = P.plain_linear(a.to(F64), w.to(F64), b.to(F64), 0.25)
+    _close(out, want, 2e-6 * math.sqrt(K_))   # no reduced-precision matrix mode: errors of float32 sums only
+    # rows do not depend on the batch around them, bit for bit
+    one = K.gemm(a[M // 2:M // 2 + 1].to(DEV), w.to(DEV), b.to(DEV), 0.25)
+    assert torch.equal(one.cpu(), out[M // 2:M // 2 + 1].cpu())
+
+
+@pytest.mark.parametrize("M,N,K_,out_dtype", [
+    (1, 16, 32, torch.bfloat16), (1, 4608, 4096, torch.bfloat16), (8, 331, 80, torch.float32), (17, 96, 200, torch.bfloat16),
+    (33, 200, 96, torch.bfloat16), (64, 73448, 128, torch.float32), (48, 100, 2048, torch.bfloat16),
+    (7, 50, 100, torch.bfloat16),        # K no multiple of 8: the plain kernel takes it
+    (100, 176, 80, torch.bfloat16), (300, 512, 256, torch.bfloat16), (65, 40, 64, torch.float32),
+])
+def test_gemm_bfloat16(K, M, N, K_, out_dtype):
+    a, w = _rand((M, K_), 11, torch.bfloat16), _rand((N, K_), 12, torch.bfloat16)
+    alpha = 0.5 if out_dtype == torch.float32 else 1.0
+    out = K.gemm(a.to(DEV), w.to(DEV), None, alpha, out_dtype)
+    assert out.dtype == out_dtype
+    want = P.plain_linear(a.to(F64), w.to(F64), None, alpha)
+    _close(out, want, 1e-5 if out_dtype == torch.float32 else 6e-3)
+    if M <= 64:
+        b = _rand((N,), 13, torch.bfloat16)
+        out = K.gemm(a.to(DEV), w.to(DEV), b.to(DEV), 0.5, out_dtype)
+        _close(out, P.plain_linear(a.to(F64), w.to(F64), b.to(F64), 0.5), 1e-5 if out_dtype == torch.float32 else 6e-3)
+
+
+def _paged(k, v, page, n_pages, seed, dtype):
+    """Scatters contiguous per-request keys/values [n, nkv, d] into a paged cache with a shuffled
+    block table; unused slots hold large finite garbage so that a read beyond a length shows."""
+    nkv, d = k[0].shape[1], k[0].shape[2]
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kc = torch.full((n_pages, nkv, page, d), 7.0, dtype=dtype)
+    vc = torch.full((n_pages, nkv, d, page), -9.0, dtype=dtype)
+    tables = []
+    for kr, vr in zip(k, v):
+        n = kr.shape[0]
+        tab = [perm.pop() for _ in range(-(-n // page))]
+        for i in range(n):
+            kc[tab[i // page], :, i % page, :] = kr[i].to(dtype)
+            vc[tab[i // page], :, :, i % page] = vr[i].to(dtype)
+        tables.append(tab)
+    width = max(len(t) for t in tables)
+    bt = torch.full((len(tables), width), -1, dtype=torch.int32)
+    for i, t in enumerate(tables):
+        bt[i, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    return kc, vc, bt
+
+
+def _attention_case(K, dtype, nh, nkv, d, page, lens, qlens, window=0, seed=0, spike=False):
+    """Requests with `lens[i]` cached keys of which the last `qlens[i]` are this step's queries."""
+    ks = [_rand((n, nkv, d), seed + 10 * i + 1, dtype) for i, n in enumerate(lens)]
+    vs = [_rand((n, nkv, d), seed + 10 * i + 2, dtype) for i, n in enumerate(lens)]
+    qs = [_rand((n, nh, d), seed + 10 * i + 3, dtype) for i, n in enumerate(lens)]
+    if spike:
+        # one far key per request must dominate: its score stands out by construction
+        for q, k in zip(qs, ks):
+            far = 3 if k.shape[0] > 3 else 0
+            k[far] = (q[-1, 0:1, :].float() * 4.0 / math.sqrt(d)).to(dtype)
+    n_pages = sum(-(-n // page) for n in lens) + 3
+    kc, vc, bt = _paged(ks, vs, page, n_pages, seed, dtype)
+    q_rows, seg, pos = [], [], []
+    for i, (n, ql) in enumerate(zip(lens, qlens)):
+        q_rows.append(qs[i][n - ql:])
+        seg += [i] * ql
+        pos += list(range(n - ql, n))
+    q = torch.cat(q_rows).reshape(-1, nh * d)
+    out = K.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), torch.tensor(seg, dtype=torch.int32, device=DEV),
+                            torch.tensor(pos, dtype=torch.int32, device=DEV), nh, nkv, d, 1 / math.sqrt(d), window,
+                            max_total_len=max(lens))
+    want = []
+    for i, (n, ql) in enumerate(zip(lens, qlens)):
+        full = P.plain_attention(qs[i].to(F64), ks[i].to(F64), vs[i].to(F64), 1 / math.sqrt(d), window)
+        want.append(full[n - ql:].reshape(ql, nh * d))
+    return out, torch.cat(want)
+
+
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 3, 48, 16), (5, 5, 80, 7), (2, 1, 256, 16)])
+def test_attention_float32(K, nh, nkv, d, page):
+    out, want = _attention_case(K, torch.float32, nh, nkv, d, page, lens=[1, 70, 33, 130], qlens=[1, 70, 1, 5])
+    _close(out, want, 3e-6)
+    out, want = _attention_case(K, torch.float32, nh, nkv, d, page, lens=[90, 20], qlens=[2, 20], window=11, seed=5)
+    _close(out, want, 3e-6)
+    out, want = _attention_case(K, torch.float32, nh, nkv, d, page, lens=[300, 65], qlens=[1, 1], seed=9, spike=True)
+    _close(out, want, 3e-6)
+
+
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 16), (3, 1, 32, 16), (6, 3, 48, 32), (32, 2, 128, 64), (16, 16, 64, 16),
+                                            (34, 2, 80, 16), (5, 1, 112, 48)])
+def test_attention_bfloat16_matrix_cores(K, nh, nkv, d, page):
+    # whole prompts, decode rows, a portion with history, lengths that cross key chunks of 256
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[1, 70, 33, 300], qlens=[1, 70, 1, 9])
+    _close(out, want, 1.2e-2)
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[700, 257, 256, 31], qlens=[1, 1, 1, 31], seed=3)
+    _close(out, want, 1.2e-2)
+    # a window's edge, inside a page and across chunks
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[90, 20, 600], qlens=[2, 20, 3], window=11, seed=5)
+    _close(out, want, 1.2e-2)
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[600, 40], qlens=[1, 40], window=300, seed=6)
+    _close(out, want, 1.2e-2)
+    # a far key among hundreds must dominate
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[520, 65], qlens=[1, 1], seed=9, spike=True)
+    _close(out, want, 1.2e-2)
+
+
+def test_attention_does_not_depend_on_the_batch(K):
+    """The same token alone and inside a larger batch gives the same bits (bfloat16 kernel)."""
+    nh, nkv, d, page = 8, 2, 64, 16
+    out_a, _ = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[300], qlens=[1], seed=0)
+    out_b, _ = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[300, 50, 700], qlens=[1, 50, 2], seed=0)
+    assert torch.equal(out_a.cpu()[0], out_b.cpu()[0])
+
+
+def test_argmax_and_sampling(K):
+    V = 73448
+    logits = _rand((5, V), 20, scale=3.0)
+    logits[1, 100] = logits[1, 70000] = 50.0      # a tie: the first index wins
+    logits[2, V - 1] = 60.0
+    dl = logits.to(DEV)
+    assert K.argmax(dl).tolist() == [int(torch.argmax(logits[0])), 100, V - 1, int(torch.argmax(logits[3])), int(torch.argmax(logits[4]))]
+
+    def run(temp, k, p, u, rows=logits):
+        n = rows.shape[0]
+        mk = lambda v, dt: torch.tensor([v] * n if not isinstance(v, list) else v, dtype=dt, device=DEV)
+        return K.sample(rows.to(DEV), mk(temp, torch.float32), mk(k, torch.int32), mk(p, torch.float32),
+                        mk(u, torch.float32)).tolist()
+
+    assert run(1.0, 1, 1.0, 0.5) == K.argmax(dl).tolist()           # top_k 1 is greedy
+    assert run(0.0, 0, 1.0, 0.9) == K.argmax(dl).tolist()           # temperature 0 is greedy
+    # inverse CDF in vocabulary order against the plain implementation, over many u
+    small = _rand((1, 331), 21, scale=2.0)
+    for temp, k, p in [(0.8, 0, 1.0), (1.3, 5, 1.0), (1.0, 0, 0.6), (0.7, 40, 0.9), (1.0, 331, 1.0), (2.0, 2, 0.5)]:
+        dist = P.plain_sample_distribution(small[0], temp, k, p)
+        cdf = torch.cumsum(dist, 0)
+        us = [i / 64.0 + 1 / 128.0 for i in range(64)]
+        got = run(temp, k, p, us, small.expand(64, 331).contiguous())
+        for u, tok in zip(us, got):
+            assert dist[tok] > 0, f"token {tok} is outside the kept set (T={temp}, k={k}, p={p})"
+            lo = float(cdf[tok] - dist[tok])
+            assert lo - 1e-4 <= u <= float(cdf[tok]) + 1e-4, f"u={u} not in token {tok}'s interval"
+    # frequencies over many draws follow the probabilities
+    dist = P.plain_sample_distribution(small[0], 1.0, 8, 1.0)
+    n = 4096
+    g = torch.Generator().manual_seed(1)
+    us = torch.rand(n, generator=g).tolist()
+    got = torch.tensor(run(1.0, 8, 1.0, us, small.expand(n, 331).contiguous()))
+    freq = torch.bincount(got, minlength=331).to(F64) / n
+    assert float((freq - dist).abs().max()) < 0.03
+    # the big vocabulary: top-k keeps exactly the k largest
+    top = set(torch.topk(logits[0], 3).indices.tolist())
+    for u in (0.01, 0.4, 0.99):
+        assert run(1.5, 3, 1.0, u, logits[:1])[0] in top
