@@ -1,10 +1,11 @@
 // Paged attention on the matrix cores (bfloat16 in, float softmax and accumulation).
 //
-// Same contract as attn_basic.hip.  One wave serves one token and one group of up to 16 query
-// heads that share a KV head, over one chunk of ATT_CHUNK keys; chunks are aligned to absolute key
-// index, so what is summed in which order depends on (request, position) alone.  With more than
-// one chunk the partial results (max, sum, unnormalised output) go to a workspace and a second
-// kernel merges them in chunk order.
+// Same contract as attn_basic.hip.  A workgroup of 4 waves serves one token and one group of up to
+// 16 query heads that share a KV head, over one chunk of ATT_CHUNK keys; each wave takes a quarter
+// of the chunk, the four partial results are merged through LDS.  Chunks are aligned to absolute
+// key index, so what is summed in which order depends on (request, position) alone.  With more
+// than one chunk the partial results (max, sum, unnormalised output) go to a workspace and a
+// second kernel merges them in chunk order.
 //
 // Per 32 keys:  S^T[keys x heads] = K Q^T   (v_mfma_f32_16x16x32_bf16, K rows on the A side, read
 //                                            straight from the cache; d is the reduced dimension)
@@ -13,6 +14,8 @@
 //                                            consecutive keys of one dim are one 16-byte load)
 // The rows of the two S tiles are assigned to keys so that each lane ends up with the
 // probabilities of 8 consecutive keys: they feed the second product without leaving registers.
+// All loads of a wave's 64 keys (K and V) are issued before the first product; they are
+// unconditional 16-byte loads from clamped addresses, masked afterwards.
 // Needs: head size a multiple of 16 up to 128, page size a multiple of 16.
 #include "common.h"
 
@@ -20,14 +23,21 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 #define ATT_CHUNK 256
+#define ATT_WAVES 4
+#define ATT_WKEYS (ATT_CHUNK / ATT_WAVES)  // keys per wave
+#define ATT_ITERS (ATT_WKEYS / 32)
 #define NEG_BIG (-1.0e30f)
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
     return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
 }
 
+__device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
 template <int D16>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(ATT_WAVES * 64)
 attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
                  const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                  const int* __restrict__ block_tables, const int* __restrict__ seg,
@@ -35,157 +45,229 @@ attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __re
                  int out_stride, float scale_log2e, int window, int nsplit) {
     constexpr int D = D16 * 16;
     constexpr int KS = (D + 31) / 32;
+    __shared__ float sm_acc[ATT_WAVES][D16][64][4];
+    __shared__ float sm_ml[ATT_WAVES][16][2];
     const int t = blockIdx.x;
     const int G = nh / nkv;
     const int HG = (G + 15) / 16;
     const int kvh = blockIdx.y / HG, hg = blockIdx.y % HG;
     const int split = blockIdx.z;
-    const int lane = threadIdx.x, r = lane & 15, qg = lane >> 4;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qg = lane >> 4;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int hcol = hg * 16 + r;
     const bool head_ok = hcol < G;
     const int head = kvh * G + (head_ok ? hcol : G - 1);
 
-    int k_begin = split * ATT_CHUNK;
-    int k_end = k_begin + ATT_CHUNK;
-    if (k_begin < lo) k_begin = lo;
-    if (k_end > p + 1) k_end = p + 1;
-    if (k_begin >= k_end) {
-        if (nsplit > 1 && head_ok && qg == 0) {
+    // the chunk's valid keys [c_begin, c_end); empty: nothing to do for the whole workgroup
+    int c_begin = split * ATT_CHUNK, c_end = c_begin + ATT_CHUNK;
+    if (c_begin < lo) c_begin = lo;
+    if (c_end > p + 1) c_end = p + 1;
+    if (c_begin >= c_end) {
+        if (nsplit > 1 && head_ok && qg == 0 && wave == 0) {
             float* ml = ws_ml + (((size_t)t * nh + head) * nsplit + split) * 2;
             ml[0] = NEG_BIG;
             ml[1] = 0.f;
         }
         return;
     }
+    // this wave's keys [k_begin, k_end) within the chunk (may be empty)
+    const int w_base = split * ATT_CHUNK + wave * ATT_WKEYS;
+    const int k_begin = w_base > c_begin ? w_base : c_begin;
+    const int k_end = (w_base + ATT_WKEYS < c_end) ? w_base + ATT_WKEYS : c_end;
+    const bool wave_has_keys = k_begin < k_end;
+
     const int* bt = block_tables + (size_t)seg[t] * max_blocks;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
-
-    uint4 qf[KS];
-    const bf16* qrow = q + (size_t)t * q_stride + (size_t)head * D;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        const int dofs = ks * 32 + qg * 8;
-        qf[ks] = (dofs < D) ? *reinterpret_cast<const uint4*>(qrow + dofs) : zero4;
-    }
     f32x4 acc[D16];
 #pragma unroll
     for (int db = 0; db < D16; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m = NEG_BIG, lsum = 0.f;
 
-    for (int kb = k_begin & ~31; kb < k_end; kb += 32) {
-        // ---- S^T = K Q^T for two tiles of 16 keys; row i of tile tau is key kb + (i/4)*8 + tau*4 + i%4
-        f32x4 s[2];
+    if (wave_has_keys) {
+        // Q fragments: lane (r, qg) holds dims ks*32 + qg*8 .. +8 of head column r
+        uint4 qf[KS];
+        const bf16* qrow = q + (size_t)t * q_stride + (size_t)head * D;
 #pragma unroll
-        for (int tau = 0; tau < 2; ++tau) {
-            int key = kb + (r >> 2) * 8 + tau * 4 + (r & 3);
-            key = key < k_begin ? k_begin : (key >= k_end ? k_end - 1 : key);  // stay on pages that exist
-            const int pg = bt[key / page];
-            const bf16* krow = kc + (((size_t)pg * nkv + kvh) * page + (key % page)) * D;
-            s[tau] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const int dofs = ks * 32 + qg * 8;
-                const uint4 kf = (dofs < D) ? *reinterpret_cast<const uint4*>(krow + dofs) : zero4;
-                s[tau] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
-                                                                 __builtin_bit_cast(bf16x8, qf[ks]), s[tau], 0, 0, 0);
-            }
+        for (int ks = 0; ks < KS; ++ks) {
+            const int dofs = ks * 32 + qg * 8;
+            const uint4 v = *reinterpret_cast<const uint4*>(qrow + (dofs < D ? dofs : 0));
+            qf[ks] = dofs < D ? v : zero4;
         }
-        // lane (r, qg) now holds, for head column r, keys kb + qg*8 + tau*4 + e
-        float sv[8];
-        float mx = NEG_BIG;
+        // ---- every load of this wave's keys, issued at once
+        uint4 kf[ATT_ITERS][2][KS];
+        uint4 vf[ATT_ITERS][D16];
 #pragma unroll
-        for (int tau = 0; tau < 2; ++tau)
+        for (int it = 0; it < ATT_ITERS; ++it) {
+            const int kb = w_base + it * 32;
+            // row i of S tile tau is key kb + (i/4)*8 + tau*4 + i%4; clamped onto pages that exist
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int key = kb + qg * 8 + tau * 4 + e;
-                const bool ok = key >= k_begin && key < k_end;
-                const float v = ok ? s[tau][e] * scale_log2e : NEG_BIG;
-                sv[tau * 4 + e] = v;
-                mx = fmaxf(mx, v);
+            for (int tau = 0; tau < 2; ++tau) {
+                int key = kb + (r >> 2) * 8 + tau * 4 + (r & 3);
+                key = key < k_begin ? k_begin : (key >= k_end ? k_end - 1 : key);
+                const int pg = bt[key / page];
+                const bf16* krow = kc + (((size_t)pg * nkv + kvh) * page + (key % page)) * D;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const int dofs = ks * 32 + qg * 8;
+                    kf[it][tau][ks] = *reinterpret_cast<const uint4*>(krow + (dofs < D ? dofs : 0));
+                }
             }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m, mx);
-        const float corr = __builtin_amdgcn_exp2f(m - m_new);
-        float pe[8];
-        float rs = 0.f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            pe[j] = (sv[j] > 0.5f * NEG_BIG) ? __builtin_amdgcn_exp2f(sv[j] - m_new) : 0.f;
-            rs += pe[j];
-        }
-        rs += __shfl_xor(rs, 16, 64);
-        rs += __shfl_xor(rs, 32, 64);
-        lsum = lsum * corr + rs;
-        m = m_new;
-        uint4 pf;
-        pf.x = pack_bf16x2(pe[0], pe[1]);
-        pf.y = pack_bf16x2(pe[2], pe[3]);
-        pf.z = pack_bf16x2(pe[4], pe[5]);
-        pf.w = pack_bf16x2(pe[6], pe[7]);
-        // ---- O^T += V^T P^T; this lane's 8 keys are kb + qg*8 .. +8, on one page
-        const int key0 = kb + qg * 8;
-        const bool vok = key0 < k_end && key0 + 8 > k_begin;
-        const bf16* vbase = nullptr;
-        if (vok) {
+            // this lane's 8 keys of the second product are kb + qg*8 .. +8 (one page); a group with no
+            // valid key is read from the wave's first valid group instead and masked below
+            int key0 = kb + qg * 8;
+            if (key0 >= k_end || key0 + 8 <= k_begin) key0 = k_begin & ~7;
             const int pg = bt[key0 / page];
-            vbase = vc + ((size_t)pg * nkv + kvh) * D * page + (key0 % page);
+            const bf16* vbase = vc + ((size_t)pg * nkv + kvh) * D * page + (key0 % page);
+#pragma unroll
+            for (int db = 0; db < D16; ++db)
+                vf[it][db] = *reinterpret_cast<const uint4*>(vbase + (size_t)(db * 16 + r) * page);
         }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int db = 0; db < D16; ++db) {
-            const uint4 vf = vok ? *reinterpret_cast<const uint4*>(vbase + (size_t)(db * 16 + r) * page) : zero4;
+        for (int it = 0; it < ATT_ITERS; ++it) {
+            const int kb = w_base + it * 32;
+            if (kb >= k_end || kb + 32 <= k_begin) continue;  // wave-uniform
+            f32x4 s[2];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[db][e] *= corr;
-            acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
-                                                             __builtin_bit_cast(bf16x8, pf), acc[db], 0, 0, 0);
+            for (int tau = 0; tau < 2; ++tau) {
+                s[tau] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const int dofs = ks * 32 + qg * 8;
+                    s[tau] = mfma16(dofs < D ? kf[it][tau][ks] : zero4, qf[ks], s[tau]);
+                }
+            }
+            // lane (r, qg) holds, for head column r, keys kb + qg*8 + tau*4 + e
+            float sv[8];
+            float mx = NEG_BIG;
+#pragma unroll
+            for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int key = kb + qg * 8 + tau * 4 + e;
+                    const bool ok = key >= k_begin && key < k_end;
+                    const float v = ok ? s[tau][e] * scale_log2e : NEG_BIG;
+                    sv[tau * 4 + e] = v;
+                    mx = fmaxf(mx, v);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m, mx);
+            const float corr = __builtin_amdgcn_exp2f(m - m_new);
+            float pe[8];
+            float rs = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                pe[j] = (sv[j] > 0.5f * NEG_BIG) ? __builtin_amdgcn_exp2f(sv[j] - m_new) : 0.f;
+                rs += pe[j];
+            }
+            rs += __shfl_xor(rs, 16, 64);
+            rs += __shfl_xor(rs, 32, 64);
+            lsum = lsum * corr + rs;
+            m = m_new;
+            uint4 pf;
+            pf.x = pack_bf16x2(pe[0], pe[1]);
+            pf.y = pack_bf16x2(pe[2], pe[3]);
+            pf.z = pack_bf16x2(pe[4], pe[5]);
+            pf.w = pack_bf16x2(pe[6], pe[7]);
+            const int key0 = kb + qg * 8;
+            const bool vok = key0 < k_end && key0 + 8 > k_begin;  // else the loaded values are another group's
+#pragma unroll
+            for (int db = 0; db < D16; ++db) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[db][e] *= corr;
+                acc[db] = mfma16(vok ? vf[it][db] : zero4, pf, acc[db]);
+            }
         }
     }
-    // acc[db][e] is dim db*16 + qg*4 + e of head column r
+    // ---- merge the four waves; acc[db][e] is dim db*16 + qg*4 + e of head column r
+#pragma unroll
+    for (int db = 0; db < D16; ++db) *reinterpret_cast<f32x4*>(&sm_acc[wave][db][lane][0]) = acc[db];
+    if (qg == 0) {
+        sm_ml[wave][r][0] = m;
+        sm_ml[wave][r][1] = lsum;
+    }
+    __syncthreads();
+    float M = NEG_BIG;
+#pragma unroll
+    for (int w = 0; w < ATT_WAVES; ++w) M = fmaxf(M, sm_ml[w][r][0]);
+    float wgt[ATT_WAVES];
+    float L = 0.f;
+#pragma unroll
+    for (int w = 0; w < ATT_WAVES; ++w) {
+        wgt[w] = __builtin_amdgcn_exp2f(sm_ml[w][r][0] - M);
+        L += sm_ml[w][r][1] * wgt[w];
+    }
     if (!head_ok) return;
-    if (nsplit == 1) {
-        const float inv = 1.0f / lsum;
-        bf16* orow = out + (size_t)t * out_stride + (size_t)head * D;
+    const size_t slot = ((size_t)t * nh + head) * nsplit + split;
+    for (int db = wave; db < D16; db += ATT_WAVES) {
+        f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int db = 0; db < D16; ++db) {
-            uint2 w;
-            w.x = pack_bf16x2(acc[db][0] * inv, acc[db][1] * inv);
-            w.y = pack_bf16x2(acc[db][2] * inv, acc[db][3] * inv);
-            *reinterpret_cast<uint2*>(orow + db * 16 + qg * 4) = w;
-        }
-    } else {
-        const size_t slot = ((size_t)t * nh + head) * nsplit + split;
-        float* wa = ws_acc + slot * D;
+        for (int w = 0; w < ATT_WAVES; ++w) {
+            const f32x4 a = *reinterpret_cast<const f32x4*>(&sm_acc[w][db][lane][0]);
 #pragma unroll
-        for (int db = 0; db < D16; ++db)
-            *reinterpret_cast<f32x4*>(wa + db * 16 + qg * 4) = acc[db];
-        if (qg == 0) {
-            ws_ml[slot * 2] = m;
-            ws_ml[slot * 2 + 1] = lsum;
+            for (int e = 0; e < 4; ++e) o[e] += a[e] * wgt[w];
         }
+        if (nsplit == 1) {
+            const float inv = 1.0f / L;
+            uint2 wv;
+            wv.x = pack_bf16x2(o[0] * inv, o[1] * inv);
+            wv.y = pack_bf16x2(o[2] * inv, o[3] * inv);
+            *reinterpret_cast<uint2*>(out + (size_t)t * out_stride + (size_t)head * D + db * 16 + qg * 4) = wv;
+        } else {
+            *reinterpret_cast<f32x4*>(ws_acc + slot * D + db * 16 + qg * 4) = o;
+        }
+    }
+    if (nsplit > 1 && wave == 0 && qg == 0) {
+        ws_ml[slot * 2] = M;
+        ws_ml[slot * 2 + 1] = L;
     }
 }
 
-// out[t, h, :] = sum_i acc_i 2^(m_i - M) / sum_i l_i 2^(m_i - M), chunks in ascending order
+// out[t, h, :] = sum_i acc_i 2^(m_i - M) / sum_i l_i 2^(m_i - M), chunks in ascending order.
+// One wave per (token, head); lanes first share the chunks' (m, l), then each sums its dims.
 __global__ void __launch_bounds__(64)
 attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
                   const int* __restrict__ pos, int nh, int D, int out_stride, int window, int nsplit) {
+    __shared__ float wsm[64];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int s_lo = lo / ATT_CHUNK, s_hi = p / ATT_CHUNK;
     const size_t base = ((size_t)t * nh + h) * nsplit;
-    float M = NEG_BIG;
-    for (int s = s_lo; s <= s_hi; ++s) M = fmaxf(M, ws_ml[(base + s) * 2]);
-    float L = 0.f;
-    for (int s = s_lo; s <= s_hi; ++s) L += ws_ml[(base + s) * 2 + 1] * __builtin_amdgcn_exp2f(ws_ml[(base + s) * 2] - M);
+    float o[4] = {0.f, 0.f, 0.f, 0.f};  // dims lane, lane+64, ... (D <= 256)
+    float M = NEG_BIG, L = 0.f;
+    // chunks in groups of 64: running rescale keeps one pass
+    for (int g0 = s_lo; g0 <= s_hi; g0 += 64) {
+        const int s = g0 + lane;
+        const bool ok = s <= s_hi;
+        const float ms = ok ? ws_ml[(base + s) * 2] : NEG_BIG;
+        const float ls = ok ? ws_ml[(base + s) * 2 + 1] : 0.f;
+        const float Mn = fmaxf(M, wave_max(ms));
+        const float corr = __builtin_amdgcn_exp2f(M - Mn);
+        const float w = __builtin_amdgcn_exp2f(ms - Mn);
+        L = L * corr + wave_sum(ls * w);
+        M = Mn;
+        __syncthreads();
+        wsm[lane] = w;
+        __syncthreads();
+        const int cnt = (s_hi - g0 + 1 < 64) ? s_hi - g0 + 1 : 64;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int dd = lane + 64 * i;
+            if (dd < D) {
+                float a = o[i] * corr;
+                for (int j = 0; j < cnt; ++j) a += ws_acc[(base + g0 + j) * D + dd] * wsm[j];
+                o[i] = a;
+            }
+        }
+    }
     const float inv = 1.0f / L;
-    for (int dd = lane; dd < D; dd += 64) {
-        float o = 0.f;
-        for (int s = s_lo; s <= s_hi; ++s)
-            o += ws_acc[(base + s) * D + dd] * __builtin_amdgcn_exp2f(ws_ml[(base + s) * 2] - M);
-        out[(size_t)t * out_stride + (size_t)h * D + dd] = from_f32<bf16>(o * inv);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int dd = lane + 64 * i;
+        if (dd < D) out[(size_t)t * out_stride + (size_t)h * D + dd] = from_f32<bf16>(o[i] * inv);
     }
 }
 
@@ -207,10 +289,10 @@ extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q
     const float sl2 = scale * 1.4426950408889634f;
 #define AM_CASE(D16)                                                                                           \
     case D16:                                                                                                  \
-        attn_mfma_kernel<D16><<<grid, 64, 0, stream>>>((bf16*)out, (float*)ws_acc, (float*)ws_ml, (const bf16*)q, \
-                                                       (const bf16*)kc, (const bf16*)vc, (const int*)block_tables, \
-                                                       (const int*)seg, (const int*)pos, nh, nkv, page, max_blocks, \
-                                                       q_stride, out_stride, sl2, window, nsplit);             \
+        attn_mfma_kernel<D16><<<grid, ATT_WAVES * 64, 0, stream>>>(                                            \
+            (bf16*)out, (float*)ws_acc, (float*)ws_ml, (const bf16*)q, (const bf16*)kc, (const bf16*)vc,      \
+            (const int*)block_tables, (const int*)seg, (const int*)pos, nh, nkv, page, max_blocks, q_stride,  \
+            out_stride, sl2, window, nsplit);                                                                  \
         break
     switch (d / 16) {
         AM_CASE(1); AM_CASE(2); AM_CASE(3); AM_CASE(4); AM_CASE(5); AM_CASE(6); AM_CASE(7); AM_CASE(8);

@@ -1,78 +1,117 @@
 // C[M,N] = alpha * (X[M,K] W[N,K]^T + bias) for few rows of X (M <= 64), bfloat16 in, float
 // accumulation: the decode-side projection, bound by reading W once from HBM.
 //
-// One workgroup of 8 waves owns 16 rows of W (16 outputs for every token).  The waves split K into
-// 8 contiguous slices; each streams its slice of the 16 rows straight from global memory into MFMA
-// operands (v_mfma_f32_16x16x32_bf16: W rows on the A side, tokens on the B side, 16 tokens per
-// accumulator, up to 4 accumulators), with every load of a chunk issued before the chunk's first
-// MFMA.  The 8 partial tiles are summed through LDS in wave order, so the result is deterministic.
-// The X fragments come from L2 (X is at most 64 x K).
+// v_mfma_f32_16x16x32_bf16 with W rows on the A side and tokens on the B side: one accumulator is
+// 16 outputs x 16 tokens.  The waves of a workgroup split K into contiguous slices and stream
+// their slice of the workgroup's W rows straight from global memory into MFMA operands; the
+// partial tiles are summed through LDS in wave order, so the result is deterministic.
+//
+// Two kernels:
+//  * stream:  RT tiles of 16 W rows per workgroup, up to 4 token groups; the X fragments are
+//             re-read from L2 for every workgroup.  Any K (multiple of 8), any M <= 64.
+//  * resident (M <= 16, K <= 16 waves * KSTEPS * 32): each wave keeps the X fragments of its
+//             K slice in registers and the workgroup walks over W row tiles, prefetching the next
+//             tile's rows while the current one is reduced; X is read once per workgroup.
 // K must be a multiple of 8 (16-byte loads); rows of X and W must be 16-byte aligned.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-#define SK_WAVES 8
-#define SK_UNROLL 4
 
-template <int MG, typename TC>
-__global__ void __launch_bounds__(SK_WAVES * 64)
-gemm_skinny_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
-                   const bf16* __restrict__ bias, int M, int N, int K, int lda, int ldw, int ldc,
-                   float alpha) {
-    __shared__ float part[SK_WAVES][MG][64][4];
+__device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+template <int WAVES, int MG, int RT, int UNROLL, typename TC>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_skinny_stream_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
+                          const bf16* __restrict__ bias, int M, int N, int K, int lda, int ldw, int ldc,
+                          float alpha) {
+    __shared__ float part[WAVES][RT][MG][64][4];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, q = lane >> 4;
-    const int n0 = blockIdx.x * 16;
+    const int n0 = blockIdx.x * (16 * RT);
     const int steps_total = (K + 31) >> 5;
-    const int per = (steps_total + SK_WAVES - 1) / SK_WAVES;
+    const int per = (steps_total + WAVES - 1) / WAVES;
     const int s0 = wave * per;
     const int s1 = (s0 + per < steps_total) ? s0 + per : steps_total;
 
-    const int wrow = (n0 + r < N) ? n0 + r : N - 1;
-    const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)wrow * ldw);
+    const uint4* wp[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        const int row = (n0 + t * 16 + r < N) ? n0 + t * 16 + r : N - 1;
+        wp[t] = reinterpret_cast<const uint4*>(W + (size_t)row * ldw);
+    }
     const uint4* xp[MG];
+    bool xok[MG];
 #pragma unroll
     for (int g = 0; g < MG; ++g) {
-        const int m = (g * 16 + r < M) ? g * 16 + r : M - 1;
-        xp[g] = reinterpret_cast<const uint4*>(X + (size_t)m * lda);
+        xok[g] = g * 16 + r < M;
+        xp[g] = reinterpret_cast<const uint4*>(X + (size_t)(xok[g] ? g * 16 + r : 0) * lda);
     }
-    f32x4 acc[MG];
+    f32x4 acc[RT][MG];
 #pragma unroll
-    for (int g = 0; g < MG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int g = 0; g < MG; ++g) acc[t][g] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // Loads are unconditional 16-byte loads from clamped (always valid) addresses; what lies beyond K,
+    // beyond this wave's slice or beyond M is replaced by zeros afterwards.  (A conditional load
+    // would be split into four 4-byte loads behind branches.)  The chunk after the one being
+    // multiplied is already on its way.
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-    for (int s = s0; s < s1; s += SK_UNROLL) {
-        uint4 a[SK_UNROLL];
-        uint4 b[SK_UNROLL][MG];
+    const int k8_last = (K >> 3) - 1;
+    uint4 a[2][UNROLL][RT];
+    uint4 b[2][UNROLL][MG];
+    auto load_chunk = [&](int s, int buf) {
 #pragma unroll
-        for (int u = 0; u < SK_UNROLL; ++u) {
+        for (int u = 0; u < UNROLL; ++u) {
             const int k8 = (s + u) * 4 + q;  // index of this lane's group of 8 elements
-            const bool ok = (s + u < s1) && (k8 * 8 + 8 <= K);
-            a[u] = ok ? wp[k8] : zero;
+            const int k8c = k8 < k8_last ? k8 : k8_last;
 #pragma unroll
-            for (int g = 0; g < MG; ++g) b[u][g] = ok ? xp[g][k8] : zero;
+            for (int t = 0; t < RT; ++t) a[buf][u][t] = wp[t][k8c];
+#pragma unroll
+            for (int g = 0; g < MG; ++g) b[buf][u][g] = xp[g][k8c];
         }
+    };
+    auto mul_chunk = [&](int s, int buf) {
 #pragma unroll
-        for (int u = 0; u < SK_UNROLL; ++u)
+        for (int u = 0; u < UNROLL; ++u) {
+            const int k8 = (s + u) * 4 + q;
+            const bool ok = (s + u < s1) && (k8 <= k8_last);
 #pragma unroll
-            for (int g = 0; g < MG; ++g)
-                acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[u]),
-                                                                 __builtin_bit_cast(bf16x8, b[u][g]), acc[g], 0, 0, 0);
+            for (int t = 0; t < RT; ++t)
+#pragma unroll
+                for (int g = 0; g < MG; ++g)
+                    acc[t][g] = mfma16(ok ? a[buf][u][t] : zero, xok[g] ? b[buf][u][g] : zero, acc[t][g]);
+        }
+    };
+    if (s0 < s1) load_chunk(s0, 0);
+    for (int s = s0; s < s1; s += 2 * UNROLL) {
+        if (s + UNROLL < s1) load_chunk(s + UNROLL, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mul_chunk(s, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s + 2 * UNROLL < s1) load_chunk(s + 2 * UNROLL, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s + UNROLL < s1) mul_chunk(s + UNROLL, 1);
+        __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
-    for (int g = 0; g < MG; ++g)
+    for (int t = 0; t < RT; ++t)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) part[wave][g][lane][e] = acc[g][e];
+        for (int g = 0; g < MG; ++g)
+            *reinterpret_cast<f32x4*>(&part[wave][t][g][lane][0]) = acc[t][g];
     __syncthreads();
-    // acc[g][e] of lane (r, q) is output row n0 + q*4 + e for token g*16 + r
-    for (int idx = threadIdx.x; idx < MG * 64 * 4; idx += SK_WAVES * 64) {
-        const int e = idx & 3, l = (idx >> 2) & 63, g = idx >> 8;
+    // acc[t][g][e] of lane (r, q) is output row n0 + t*16 + q*4 + e for token g*16 + r
+    for (int idx = threadIdx.x; idx < RT * MG * 64 * 4; idx += WAVES * 64) {
+        const int e = idx & 3, l = (idx >> 2) & 63, tg = idx >> 8;
+        const int t = tg / MG, g = tg % MG;
         float v = 0.f;
 #pragma unroll
-        for (int w = 0; w < SK_WAVES; ++w) v += part[w][g][l][e];
-        const int n = n0 + (l >> 4) * 4 + e;
+        for (int w = 0; w < WAVES; ++w) v += part[w][t][g][l][e];
+        const int n = n0 + t * 16 + (l >> 4) * 4 + e;
         const int m = g * 16 + (l & 15);
         if (n < N && m < M) {
             if (bias != nullptr) v += to_f32(bias[n]);
@@ -81,31 +120,151 @@ gemm_skinny_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* _
     }
 }
 
+// M <= 16.  WAVES waves of KSTEPS k-steps (32 elements each) cover K; X fragments stay in registers.
+template <int WAVES, int KSTEPS, typename TC>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_skinny_resident_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
+                            const bf16* __restrict__ bias, int M, int N, int K, int lda, int ldw, int ldc,
+                            float alpha, int ntiles) {
+    __shared__ float part[2][WAVES][64][4];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = lane & 15, q = lane >> 4;
+    const int s0 = wave * KSTEPS;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    const int k8_last = (K >> 3) - 1;
+    uint4 xf[KSTEPS];
+    int k8c[KSTEPS];
+    {
+        const uint4* xp = reinterpret_cast<const uint4*>(X + (size_t)(r < M ? r : 0) * lda);
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u) {
+            const int k8 = (s0 + u) * 4 + q;
+            k8c[u] = k8 < k8_last ? k8 : k8_last;
+            const uint4 v = xp[k8c[u]];
+            // zero fragments beyond K or beyond M make the clamped W loads harmless
+            xf[u] = (k8 <= k8_last && r < M) ? v : zero;
+        }
+    }
+    uint4 a[KSTEPS];
+    int tile = blockIdx.x;
+    if (tile < ntiles) {
+        const int row = (tile * 16 + r < N) ? tile * 16 + r : N - 1;
+        const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)row * ldw);
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
+    }
+    int buf = 0;
+    for (; tile < ntiles; tile += gridDim.x) {
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u) acc = mfma16(a[u], xf[u], acc);
+        // the next tile's rows are on their way while this one is reduced
+        const int next = tile + gridDim.x;
+        __builtin_amdgcn_sched_barrier(0);
+        if (next < ntiles) {
+            const int row = (next * 16 + r < N) ? next * 16 + r : N - 1;
+            const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)row * ldw);
+#pragma unroll
+            for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        *reinterpret_cast<f32x4*>(&part[buf][wave][lane][0]) = acc;
+        __syncthreads();
+        if (threadIdx.x < 256) {
+            const int e = threadIdx.x & 3, l = threadIdx.x >> 2;
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) v += part[buf][w][l][e];
+            const int n = tile * 16 + (l >> 4) * 4 + e;
+            const int m = l & 15;
+            if (n < N && m < M) {
+                if (bias != nullptr) v += to_f32(bias[n]);
+                C[(size_t)m * ldc + n] = from_f32<TC>(alpha * v);
+            }
+        }
+        buf ^= 1;  // the other buffer is free: its readers passed the barrier above one tile ago
+    }
+}
+
+static int g_num_cus = 0;
+
+static int num_cus() {
+    if (g_num_cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            g_num_cus = prop.multiProcessorCount;
+        if (g_num_cus <= 0) g_num_cus = 256;
+    }
+    return g_num_cus;
+}
+
+// variant: 0 = choose; 4 = resident; 1, 2, 3, 5, 6 = shapes of the stream kernel (see below)
 extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void* bias, int M, int N,
-                               int K, int lda, int ldw, int ldc, float alpha, int out_dtype,
+                               int K, int lda, int ldw, int ldc, float alpha, int out_dtype, int variant,
                                hipStream_t stream) {
     ILM_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: needs 1 <= M <= 64, got M=%d N=%d K=%d", M, N, K);
     ILM_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_skinny: K=%d lda=%d ldw=%d must be multiples of 8",
                 K, lda, ldw);
     ILM_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_skinny: operands must be 16-byte aligned");
     ILM_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_skinny: strides too small");
-    const int grid = (N + 15) / 16;
+    ILM_REQUIRE(out_dtype == ILM_DTYPE_BF16 || out_dtype == ILM_DTYPE_F32, "gemm_skinny: unknown output dtype %d", out_dtype);
     const int mg = (M + 15) / 16;
-#define SK_CASE(MG, TC)                                                                                   \
-    gemm_skinny_kernel<MG, TC><<<grid, SK_WAVES * 64, 0, stream>>>((TC*)C, (const bf16*)X, (const bf16*)W, \
-                                                                   (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha)
-#define SK_DISPATCH(TC)             \
-    switch (mg) {                   \
-        case 1: SK_CASE(1, TC); break; \
-        case 2: SK_CASE(2, TC); break; \
-        case 3: SK_CASE(3, TC); break; \
-        default: SK_CASE(4, TC); break; \
+    const int ksteps = (K + 31) / 32;
+    const bool can_resident = M <= 16 && ksteps <= 16 * 16;
+    // measured on MI355X at the 8B shapes: resident wins for M <= 16 where it applies, the 16-wave
+    // stream shape for long K, two row tiles when X has more than 16 rows and W is tall
+    if (variant == 0) variant = can_resident ? 4 : (M <= 16 ? 3 : (N >= 8192 ? 2 : 1));
+    if (variant == 4) {
+        ILM_REQUIRE(can_resident, "gemm_skinny: the resident kernel needs M <= 16 and K <= 8192");
+        const int ntiles = (N + 15) / 16;
+#define SR_CASE(WV, KS, TC)                                                                                 \
+    {                                                                                                       \
+        const int grid = ntiles < num_cus() * (WV == 16 ? 1 : 2) ? ntiles : num_cus() * (WV == 16 ? 1 : 2); \
+        gemm_skinny_resident_kernel<WV, KS, TC><<<grid, WV * 64, 0, stream>>>(                              \
+            (TC*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha, ntiles); \
     }
-    if (out_dtype == ILM_DTYPE_BF16) { SK_DISPATCH(bf16) }
-    else if (out_dtype == ILM_DTYPE_F32) { SK_DISPATCH(float) }
-    else ILM_REQUIRE(false, "gemm_skinny: unknown output dtype %d", out_dtype);
-#undef SK_DISPATCH
+#define SR_DISPATCH(TC)                                   \
+    if (ksteps <= 8 * 4) SR_CASE(8, 4, TC)                \
+    else if (ksteps <= 8 * 8) SR_CASE(8, 8, TC)           \
+    else if (ksteps <= 16 * 8) SR_CASE(16, 8, TC)         \
+    else SR_CASE(16, 16, TC)
+        if (out_dtype == ILM_DTYPE_BF16) { SR_DISPATCH(bf16) } else { SR_DISPATCH(float) }
+#undef SR_DISPATCH
+#undef SR_CASE
+        ILM_LAUNCH_CHECK("gemm_skinny_resident");
+        return 0;
+    }
+    // variants of the stream kernel: (waves, row tiles, unroll)
+    int wv = 8, rt = 1, unroll = 4;
+    if (variant == 2) rt = 2;
+    else if (variant == 3) { wv = 16; unroll = 2; }
+    else if (variant == 5) { wv = 16; rt = 2; unroll = 2; }
+    else if (variant == 6) { wv = 16; unroll = 4; }
+    else ILM_REQUIRE(variant == 1, "gemm_skinny: unknown variant %d", variant);
+    if (mg > 2 && wv == 16 && rt == 2) wv = 8;  // LDS for the partial tiles
+    const int grid = (N + 16 * rt - 1) / (16 * rt);
+#define SK_CASE(WV, MG, RT, U, TC)                                                                          \
+    gemm_skinny_stream_kernel<WV, MG, RT, U, TC><<<grid, WV * 64, 0, stream>>>(                             \
+        (TC*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha)
+#define SK_MG(WV, RT, U, TC)                    \
+    switch (mg) {                               \
+        case 1: SK_CASE(WV, 1, RT, U, TC); break; \
+        case 2: SK_CASE(WV, 2, RT, U, TC); break; \
+        case 3: SK_CASE(WV, 3, RT, U, TC); break; \
+        default: SK_CASE(WV, 4, RT, U, TC); break; \
+    }
+#define SK_SHAPE(TC)                                              \
+    if (wv == 8 && rt == 1) { SK_MG(8, 1, 4, TC) }                \
+    else if (wv == 8 && rt == 2) { SK_MG(8, 2, 4, TC) }           \
+    else if (wv == 16 && rt == 1 && unroll == 2) { SK_MG(16, 1, 2, TC) } \
+    else if (wv == 16 && rt == 1) { SK_MG(16, 1, 4, TC) }         \
+    else if (mg == 1) { SK_CASE(16, 1, 2, 2, TC); }               \
+    else { SK_CASE(16, 2, 2, 2, TC); }
+    if (out_dtype == ILM_DTYPE_BF16) { SK_SHAPE(bf16) } else { SK_SHAPE(float) }
+#undef SK_SHAPE
+#undef SK_MG
 #undef SK_CASE
-    ILM_LAUNCH_CHECK("gemm_skinny");
+    ILM_LAUNCH_CHECK("gemm_skinny_stream");
     return 0;
 }

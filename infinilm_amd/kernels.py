@@ -20,6 +20,7 @@ _DT = {torch.float32: 0, torch.bfloat16: 1}
 ATT_CHUNK = 256  # keys per chunk of the matrix-core attention kernel (ilm_attn_mfma_chunk())
 # INFINILM_AMD_BASIC=1 runs the plain kernels everywhere (for telling a kernel's fault from the engine's)
 FORCE_BASIC = os.environ.get("INFINILM_AMD_BASIC", "0") == "1"
+SKINNY_VARIANT = int(os.environ.get("INFINILM_AMD_SKINNY_VARIANT", "0"))  # 0: the kernel chooses
 USE_LIBRARY_GEMM = os.environ.get("INFINILM_AMD_LIBRARY_GEMM", "1") == "1"
 
 
@@ -169,7 +170,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
             and w.data_ptr() % 16 == 0
         if M <= 64 and aligned:
             _run("ilm_gemm_skinny", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
-                 w.stride(0), out.stride(0), float(alpha), _DT[out_dtype], _stream())
+                 w.stride(0), out.stride(0), float(alpha), _DT[out_dtype], SKINNY_VARIANT, _stream())
             return out
         if M > 64 and bias is None and alpha == 1.0 and out_dtype == BF16 and USE_LIBRARY_GEMM:
             # large products go to the vendor library, as the reference's linear layers do
