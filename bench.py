@@ -55,6 +55,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=32, help="layers to run (the 8B configuration has 32)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=64)
+    ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step eagerly")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -84,7 +85,8 @@ def main() -> int:
     ps = args.page_size
     pages_per_req = -(-(args.context + 1) // ps)
     num_pages = max(max_b * pages_per_req, -(-args.prefill_tokens // ps)) + 4
-    runner = make_runner(model, num_pages=num_pages, page_size=ps, max_requests=max_b + 1)
+    runner = make_runner(model, num_pages=num_pages, page_size=ps, max_requests=max_b + 1,
+                         enable_graph=not args.no_graph)
     cache = runner.cache
     for e in cache.k:
         cache.k[e].normal_(0, 1.0)

@@ -55,7 +55,8 @@ def load_model(model_dir: str, dtype=None, device="cuda:0") -> CausalLM:
     return model
 
 
-def make_runner(model: CausalLM, num_pages: int, page_size: int, max_requests: int) -> StepRunner:
+def make_runner(model: CausalLM, num_pages: int, page_size: int, max_requests: int,
+                enable_graph: bool = False) -> StepRunner:
     cache = CacheManager(model.cache_needs, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
                          dtype=model.dtype, device=model.device)
-    return StepRunner(model, cache)
+    return StepRunner(model, cache, enable_graph=enable_graph)

@@ -60,10 +60,13 @@ class StepBatch:
 class StepRunner:
     """Owns the model and the cache manager; `step()` is the one function that advances requests."""
 
-    def __init__(self, model, cache: CacheManager):
+    def __init__(self, model, cache: CacheManager, enable_graph: bool = False):
         self.model = model
         self.cache = cache
         self.device = model.device
+        self.enable_graph = bool(enable_graph)
+        self._graphs: Dict = {}          # (requests, block-table width) -> (graph, batch, logits, buffer)
+        self._graph_pool = None
         self._pinned: Optional[torch.Tensor] = None
         self._copy_done: Optional[torch.cuda.Event] = None
         self.steps = 0
@@ -77,8 +80,13 @@ class StepRunner:
             self._pinned = torch.empty((max(n, 4096) * 2,), dtype=torch.int32, pin_memory=self.device.type == "cuda")
         return self._pinned[:n]
 
-    def build_batch(self, entries: Sequence[StepEntry]) -> StepBatch:
-        """Reserves pages for every entry (all or nothing) and lays the step's metadata out."""
+    def build_batch(self, entries: Sequence[StepEntry], min_blocks: int = 0,
+                    device_buffer: Optional[torch.Tensor] = None) -> StepBatch:
+        """Reserves pages for every entry and lays the step's metadata out.
+
+        `min_blocks` pads the block tables to a fixed width and `device_buffer` receives the
+        metadata instead of a fresh tensor: a captured graph reads the same addresses at every
+        replay."""
         cache = self.cache
         V = self.model.spec.vocab_size
         if not entries:
@@ -118,7 +126,7 @@ class StepRunner:
         np.cumsum(lens, out=offsets[1:])
         G = len(cache.groups)
         ps = cache.page_size
-        max_blocks = [max(1, max(len(cache.table(e.req_id, g)) for e in entries)) for g in range(G)]
+        max_blocks = [max(1, min_blocks, max(len(cache.table(e.req_id, g)) for e in entries)) for g in range(G)]
         n_want = sum(len(e.want) for e in entries)
 
         # layout of the one int32 buffer
@@ -171,7 +179,12 @@ class StepRunner:
                     raise RuntimeError(f"request {e.req_id!r}: a new token falls on a page already given back")
                 sl[offsets[i]:offsets[i + 1]] = pages * ps + p % ps
 
-        dev = torch.empty((total,), dtype=torch.int32, device=self.device)
+        if device_buffer is None:
+            dev = torch.empty((total,), dtype=torch.int32, device=self.device)
+        else:
+            if device_buffer.numel() < total:
+                raise RuntimeError("the graph's metadata buffer is too small for this step")
+            dev = device_buffer[:total]
         dev.copy_(host, non_blocking=True)
         if self.device.type == "cuda":
             self._copy_done = torch.cuda.Event()
@@ -201,7 +214,13 @@ class StepRunner:
     # ---- the step -----------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry], taps: Optional[dict] = None) -> torch.Tensor:
         """Runs the entries' tokens as one batch and returns float32 logits [wanted, vocab] in the
-        order of the entries and of each entry's `want`."""
+        order of the entries and of each entry's `want`.
+
+        With `enable_graph`, a step of single decoded tokens that wants each token's logits replays
+        a captured HIP graph; the returned tensor is then the graph's output buffer, valid until
+        the next such step."""
+        if self.enable_graph and taps is None and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            return self._graph_step(entries)
         batch = self.build_batch(entries)
         batch.taps = taps
         logits = self.model.forward(batch, self.cache)
@@ -210,3 +229,48 @@ class StepRunner:
         self.steps += 1
         self.tokens += batch.T
         return logits
+
+    # ---- decode steps as captured graphs ----------------------------------------------------------
+    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """One graph per (number of requests, block-table width).  The width is rounded up to a power
+        of two, so a graph serves every context up to width * page tokens; the kernels' grids are
+        sized for that bound and bound their reads by each request's own length.  Between replays
+        only the metadata buffer changes (token ids, positions, slots, block tables).
+        Reference: csrc/engine/compiler/paged_compiler.cpp:59-260 (one graph per decode batch size,
+        inputs copied into captured buffers)."""
+        cache = self.cache
+        R = len(entries)
+        need = max(-(-(cache.length(e.req_id) + 1) // cache.page_size) for e in entries)
+        width = 4
+        while width < need:
+            width *= 2
+        key = (R, width)
+        slot = self._graphs.get(key)
+        if slot is None:
+            buf = torch.zeros((self._graph_buffer_size(R, width),), dtype=torch.int32, device=self.device)
+            batch = self.build_batch(entries, min_blocks=width, device_buffer=buf)
+            batch.max_total_len = width * cache.page_size     # grids are sized for the bound, not for this step
+            self.model.forward(batch, cache)                  # warm-up outside the capture; idempotent
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                logits = self.model.forward(batch, cache)
+            self._graphs[key] = (graph, batch, logits, buf)
+        else:
+            graph, batch, logits, buf = slot
+            fresh = self.build_batch(entries, min_blocks=width, device_buffer=buf)
+            if fresh.T != batch.T or fresh.block_tables[0].shape != batch.block_tables[0].shape:
+                raise RuntimeError("a decode step does not fit the graph captured for its size")
+        graph.replay()
+        for e in entries:
+            cache.commit(e.req_id, 1)
+        self.steps += 1
+        self.tokens += R
+        return logits
+
+    def _graph_buffer_size(self, R: int, width: int) -> int:
+        G = len(self.cache.groups)
+        pad = lambda n: (n + 3) // 4 * 4
+        return 3 * pad(R) + pad(R + 1) + 5 * pad(R) + G * (pad(R) + pad(R * width)) + 64

@@ -67,7 +67,8 @@ class LLM:
             model = load_model(model_path, dtype, dev)
         self.model = model
         self.default_sampling = SamplingParams(temperature=temperature, top_p=top_p, top_k=top_k, max_tokens=max_tokens)
-        runner = make_runner(model, num_pages=num_blocks, page_size=block_size, max_requests=max_batch_size)
+        runner = make_runner(model, num_pages=num_blocks, page_size=block_size, max_requests=max_batch_size,
+                             enable_graph=enable_graph)
         if max_num_batched_tokens is None:
             env = os.environ.get("INFINILM_MAX_NUM_BATCHED_TOKENS")  # python/infinilm/llm/llm.py:99-102
             max_num_batched_tokens = int(env) if env else model.spec.max_positions

@@ -1,0 +1,225 @@
+"""The engine above the step function: greedy generation through the entry point against the plain
+implementation, seeded sampling, long decoding, the first tokens of a sequence, decode steps as
+captured graphs against eager steps, preemption under a tiny pool, and the replay program itself."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_minicpm4 as P
+from helpers import CONFIGS, TOL, Driver, make_model_dir, random_tokens, rel_err
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name in ("A", "B", "C"):
+        for dtype in ("float32", "bfloat16"):
+            cfg = CONFIGS[name]()
+            d = str(tmp_path_factory.mktemp(f"eng_{name}_{dtype}"))
+            out[(name, dtype)] = (cfg, d, make_model_dir(d, cfg, seed=40 + ord(name), store=dtype))
+    return out
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_greedy_generation_through_the_entry_point(models, name):
+    """Batch of prompts of lengths 1..40, cut into portions under a small token budget and decoded
+    beside each other: the tokens equal the plain implementation's greedy tokens."""
+    from infinilm_amd import LLM, SamplingParams
+
+    cfg, d, W = models[(name, "float32")]
+    prompts = [random_tokens(cfg, n, 300 + n) for n in (1, 2, 17, 40, 9)]
+    llm = LLM(d, dtype="float32", num_blocks=24, block_size=8, max_batch_size=3, max_num_batched_tokens=11, chunk_size=7)
+    outs = llm.generate(prompt_token_ids=prompts, sampling_params=SamplingParams(top_k=1, max_tokens=16))
+    for p, o in zip(prompts, outs):
+        assert o.finished and o.finish_reason.value == "length"
+        assert o.outputs[0].token_ids == P.plain_greedy(cfg, W, p, 16), f"prompt of {len(p)} tokens"
+    assert llm.engine.runner.cache.free_pages() == 24
+    log = llm.engine.scheduler.log
+    assert any(s["decode"] > 0 and s["portions"] for s in log), "no step mixed decoded tokens with a prompt's portion"
+    llm.close()
+
+
+def test_greedy_generation_bfloat16_with_graphs(models):
+    """bfloat16 with decode steps replayed from captured graphs gives the same tokens as eager
+    bfloat16 steps, and the plain implementation's up to near ties."""
+    from infinilm_amd import LLM, SamplingParams
+
+    cfg, d, W = models[("B", "bfloat16")]
+    prompts = [random_tokens(cfg, n, 500 + n) for n in (5, 33, 12, 70)]
+    sp = SamplingParams(top_k=1, max_tokens=40)
+    toks = {}
+    for graph in (False, True):
+        llm = LLM(d, dtype="bfloat16", num_blocks=40, block_size=16, max_batch_size=4, enable_graph=graph)
+        toks[graph] = [o.outputs[0].token_ids for o in llm.generate(prompt_token_ids=prompts, sampling_params=sp)]
+        if graph:
+            assert llm.engine.runner._graphs, "no graph was captured"
+        llm.close()
+    assert toks[True] == toks[False]
+    # Against the plain implementation: up to the first token that differs the sequences are equal;
+    # where they part, the engine's token must be an argmax within the bfloat16 tolerance (a near tie).
+    for p, t in zip(prompts, toks[True]):
+        want = P.plain_greedy(cfg, W, p, 40)
+        k = next((i for i in range(40) if t[i] != want[i]), None)
+        if k is None:
+            continue
+        row = P.plain_forward(cfg, W, p + want[:k])[-1]
+        gap = float(row.max() - row[t[k]])
+        assert gap <= TOL["bfloat16"] * max(1.0, float(row.abs().max())), \
+            f"token {k}: the engine chose {t[k]}, {gap:.3f} below the plain implementation's maximum"
+
+
+def test_graph_replays_equal_eager_steps(models):
+    """Every replay is checked against an eager step on the same state, with eager work and
+    synchronisation between the replays."""
+    from infinilm_amd.engine.loading import load_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+
+    cfg, d, W = models[("C", "bfloat16")]
+    model = load_model(d, "bfloat16", "cuda:0")
+    eager = make_runner(model, num_pages=32, page_size=16, max_requests=4)
+    graph = make_runner(model, num_pages=32, page_size=16, max_requests=4, enable_graph=True)
+    prompts = {"a": random_tokens(cfg, 37, 1), "b": random_tokens(cfg, 5, 2), "c": random_tokens(cfg, 40, 3)}
+    for r in (eager, graph):
+        for rid, p in prompts.items():
+            r.cache.admit(rid)
+            r.step([StepEntry(rid, p, [])])
+    nxt = {rid: 7 + i for i, rid in enumerate(prompts)}
+    for step in range(40):   # crosses page edges and the first block-table width
+        entries = [StepEntry(rid, [t], [0]) for rid, t in nxt.items()]
+        le = eager.step(entries).clone()
+        torch.cuda.synchronize()
+        lg = graph.step(entries)
+        assert torch.equal(le.cpu(), lg.cpu()), f"replay {step} differs from the eager step"
+        nxt = {rid: int(torch.argmax(le[i])) for i, rid in enumerate(prompts)}
+    assert len(graph._graphs) >= 2   # the context outgrew the first graph's block-table width
+
+
+def test_seeded_sampling_is_reproducible_and_independent_of_the_batch(models):
+    from infinilm_amd import LLM, SamplingParams
+
+    cfg, d, W = models[("B", "float32")]
+    prompts = [random_tokens(cfg, n, 900 + n) for n in (3, 50, 120, 8)]
+    sp = SamplingParams(temperature=0.8, top_k=0, top_p=0.9, max_tokens=12)
+    runs = []
+    for batch, budget, chunk in ((4, 256, None), (2, 17, 17), (1, 256, None)):
+        llm = LLM(d, dtype="float32", num_blocks=64, block_size=8, max_batch_size=batch, max_num_batched_tokens=budget,
+                  chunk_size=chunk, seed=123)
+        runs.append([o.outputs[0].token_ids for o in llm.generate(prompt_token_ids=prompts, sampling_params=sp)])
+        llm.close()
+    assert runs[0] == runs[1] == runs[2]
+    llm = LLM(d, dtype="float32", num_blocks=64, block_size=8, max_batch_size=4, seed=124)
+    other = [o.outputs[0].token_ids for o in llm.generate(prompt_token_ids=prompts, sampling_params=sp)]
+    llm.close()
+    assert other != runs[0]
+    greedy_like = [P.plain_greedy(cfg, W, p, 12) for p in prompts]
+    assert runs[0] != greedy_like   # it does sample
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(models, dtype):
+    """A short prompt, then every further token one by one to the end of the position table."""
+    cfg, d, W = models[("C", dtype)]
+    toks = random_tokens(cfg, 400, 77)
+    drv = Driver(d, dtype, num_pages=16, page_size=32)
+    drv.step([("r", toks[:3])])
+    for i in range(3, 400):
+        drv.step([("r", toks[i:i + 1])])
+    err = rel_err(drv.request_logits("r", 400), P.plain_forward(cfg, W, toks))
+    assert err < TOL[dtype], f"error {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(models, dtype):
+    """Prompts of one and two tokens, alone and batched, and a sequence fed from its very first
+    token one token a step."""
+    cfg, d, W = models[("B", dtype)]
+    drv = Driver(d, dtype, num_pages=8, page_size=16)
+    one, two, seq = [5], [9, 300], random_tokens(cfg, 6, 3)
+    drv.step([("one", one), ("two", two)], end=["one", "two"])
+    for i, t in enumerate(seq):
+        drv.step([("seq", [t])])
+    for rid, t in (("one", one), ("two", two), ("seq", seq)):
+        err = rel_err(drv.request_logits(rid, len(t)), P.plain_forward(cfg, W, t))
+        assert err < TOL[dtype], f"{rid}: error {err:.3e}"
+
+
+def test_preemption_recomputes_and_gives_the_same_tokens(models):
+    from infinilm_amd import LLM, SamplingParams
+
+    cfg, d, W = models[("A", "float32")]
+    prompts = [random_tokens(cfg, n, 40 + n) for n in (20, 22, 18)]
+    sp = SamplingParams(top_k=1, max_tokens=30)
+    llm = LLM(d, dtype="float32", num_blocks=14, block_size=8, max_batch_size=3, admission="optimistic")
+    outs = llm.generate(prompt_token_ids=prompts, sampling_params=sp)
+    assert llm.engine.scheduler.num_preemptions > 0, "the pool was meant to run out"
+    for p, o in zip(prompts, outs):
+        assert o.outputs[0].token_ids == P.plain_greedy(cfg, W, p, 30)
+    assert llm.engine.runner.cache.free_pages() == 14
+    llm.close()
+    # the reference's admission never preempts and gives the same tokens
+    llm = LLM(d, dtype="float32", num_blocks=14, block_size=8, max_batch_size=3, admission="reserve_full")
+    outs2 = llm.generate(prompt_token_ids=prompts, sampling_params=sp)
+    assert llm.engine.scheduler.num_preemptions == 0
+    assert [o.outputs[0].token_ids for o in outs2] == [o.outputs[0].token_ids for o in outs]
+    llm.close()
+
+
+def test_step_errors_are_loud(models):
+    from infinilm_amd.engine.loading import load_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+    from infinilm_amd.cache import OutOfPages
+
+    cfg, d, W = models[("A", "float32")]
+    model = load_model(d, "float32", "cuda:0")
+    r = make_runner(model, num_pages=2, page_size=8, max_requests=2)
+    r.cache.admit("a")
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        r.step([StepEntry("a", [cfg["vocab_size"]], [0])])
+    with pytest.raises(ValueError, match="outside its"):
+        r.step([StepEntry("a", [1, 2], [2])])
+    with pytest.raises(OutOfPages):
+        r.step([StepEntry("a", list(range(17)), [])])
+    with pytest.raises(ValueError, match="exceed the model's"):
+        r.step([StepEntry("a", [1] * (cfg["max_position_embeddings"] + 1), [])])
+    with pytest.raises(ValueError, match="twice"):
+        r.step([StepEntry("a", [1], [0]), StepEntry("a", [2], [0])])
+    assert r.cache.length("a") == 0
+    with pytest.raises(RuntimeError, match="GPU only"):
+        from infinilm_amd.engine.loading import require_gpu
+        require_gpu("cpu")
+
+
+def test_trace_run_program(models, tmp_path):
+    """bin/trace_run as a user runs it: steps on stdin, logits files out, `done <step>` lines."""
+    cfg, d, W = models[("B", "float32")]
+    a, b = random_tokens(cfg, 70, 1), random_tokens(cfg, 30, 2)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:40], "want": [0, 39]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[40:42], "want": []}, {"id": "b", "tokens": b[:29], "want": [28]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[29:], "want": [0]}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[42:], "want": list(range(28))}], "end": ["a"]},
+        {"step": 4, "entries": [{"id": "c", "tokens": b, "want": [29]}], "end": ["c"]},
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", "float32",
+                           "--out", str(out), "--max-tokens", "192"],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(5)]
+    import numpy as np
+    V = cfg["vocab_size"]
+    la, lb = P.plain_forward(cfg, W, a), P.plain_forward(cfg, W, b)
+    read = lambda i: torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V))
+    assert not (out / "1.f32").exists() or read(1).shape[0] == 1
+    assert rel_err(read(0), la[[0, 39]]) < TOL["float32"]
+    assert rel_err(read(1), lb[[28]]) < TOL["float32"]
+    assert rel_err(read(2), lb[[29]]) < TOL["float32"]
+    assert rel_err(read(3), la[42:]) < TOL["float32"]
+    assert rel_err(read(4), lb[[29]]) < TOL["float32"]
