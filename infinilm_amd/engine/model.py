@@ -84,12 +84,14 @@ class CausalLM:
             view = cache.view(run.cache, batch, run.writes_cache) if run.cache is not None else None
             self.blocks[run.layer].forward(stream, batch, view)
             if taps is not None:
-                taps[f"run{i}"] = (stream.residual.clone(), stream.pending.clone(), stream.pending_scale)
+                taps[f"run{i}"] = (stream.residual.clone(), None if stream.pending is None else stream.pending.clone(),
+                                   stream.pending_scale)
         if batch.num_wanted == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         if not batch.wants_all_rows:
             last = ResidualStream(kernels.gather_rows(stream.residual, batch.want_rows))
-            last.push(kernels.gather_rows(stream.pending, batch.want_rows), stream.pending_scale)
+            if stream.pending is not None:
+                last.push(kernels.gather_rows(stream.pending, batch.want_rows), stream.pending_scale)
             stream = last
         x = self.final_norm.forward(stream)
         return kernels.gemm(x, self.head, None, self.spec.head.scale, torch.float32)

@@ -54,6 +54,8 @@ class StepBatch:
         # host copies for parts that plan on the host
         self.h_seg_offsets: Optional[np.ndarray] = None
         self.h_start_pos: Optional[np.ndarray] = None
+        self.h_state_in: Optional[np.ndarray] = None
+        self.h_state_out: Optional[np.ndarray] = None
         self.taps: Optional[dict] = None
 
 
@@ -209,6 +211,8 @@ class StepRunner:
         b.all_decode = bool((lens == 1).all())
         b.h_seg_offsets = offsets
         b.h_start_pos = start
+        b.h_state_in = np.array(sin, dtype=np.int64)
+        b.h_state_out = np.array(sout, dtype=np.int64)
         return b
 
     # ---- the step -----------------------------------------------------------------------------

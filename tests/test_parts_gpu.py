@@ -1,0 +1,302 @@
+"""Each part of a layer alone against the plain implementation, and the generality of the parts:
+a window mixer whose pages are given back, a layer order that names a layer twice and lets a layer
+read another layer's cache, and a toy mixer with state of its own that is defined here, registered
+from here, built and stepped without a change to the framework's files."""
+import json
+import math
+import os
+
+import pytest
+import torch
+
+import plain_minicpm4 as P
+from helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F64 = torch.float64
+
+
+def _ctx(dtype):
+    from infinilm_amd.parts import BuildContext
+    return BuildContext(dtype=dtype, device=torch.device(DEV))
+
+
+def _fill(part, seed, scale=0.3):
+    g = torch.Generator().manual_seed(seed)
+    W = {}
+    for name, p in sorted(part.named_parameters().items()):
+        t = torch.randn(tuple(p.tensor.shape), generator=g) * scale
+        if t.dim() == 1:
+            t = t + 1.0
+        t = t.to(p.tensor.dtype)
+        p.tensor.copy_(t)
+        W[name] = t.to(F64)
+    return W
+
+
+class _Harness:
+    """A cache manager and step batches for one mixer, without a model around it."""
+
+    def __init__(self, needs, dtype, page_size=8, num_pages=32):
+        from infinilm_amd.cache import CacheManager
+        from infinilm_amd.engine.step import StepRunner
+
+        class _Spec:
+            vocab_size = 1 << 30
+            max_positions = 1 << 20
+
+        class _Model:
+            spec = _Spec()
+            device = torch.device(DEV)
+
+        self.cache = CacheManager(needs, page_size=page_size, num_pages=num_pages, max_requests=4, dtype=dtype, device=DEV)
+        self.runner = StepRunner(_Model(), self.cache)
+
+    def batch(self, entries):
+        from infinilm_amd.engine.step import StepEntry
+        for rid, n in entries:
+            if not self.cache.has(rid):
+                self.cache.admit(rid)
+        b = self.runner.build_batch([StepEntry(rid, [0] * n, []) for rid, n in entries])
+        return b
+
+    def commit(self, entries):
+        for rid, n in entries:
+            self.cache.commit(rid, n)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from infinilm_amd.parts import ResidualStream
+    from infinilm_amd.parts.registry import build_norm
+    from infinilm_amd.config import PartSpec
+
+    norm = build_norm(PartSpec("rmsnorm", {"size": 96, "eps": 1e-5}), _ctx(dtype))
+    W = _fill(norm, 1)
+    r = torch.randn(6, 96)
+    h = torch.randn(6, 96).to(dtype)
+    stream = ResidualStream(r.to(DEV).clone())
+    stream.push(h.to(DEV), 0.7)
+    x = norm.forward(stream)
+    assert stream.pending is None
+    want_r = r.to(F64) + 0.7 * h.to(F64)
+    assert rel_err(stream.residual, want_r) < 1e-6
+    assert rel_err(x, P.plain_rmsnorm(want_r, W["weight"], 1e-5)) < (2e-6 if dtype == torch.float32 else 1e-2)
+
+
+def test_rotary_part_tables():
+    from infinilm_amd.parts.registry import build_position_encoding
+    from infinilm_amd.config import PartSpec
+
+    for make in (P.tiny_config_a, P.tiny_config_b, P.tiny_config_c):
+        cfg = make()
+        d = P.plain_head_dim(cfg)
+        rope = build_position_encoding(PartSpec("rotary", {"head_dim": d, "rotary_dim": d,
+                                                           "max_positions": cfg["max_position_embeddings"],
+                                                           "theta": cfg["rope_theta"], "scaling": cfg.get("rope_scaling")}),
+                                       _ctx(torch.float32))
+        cos, sin = P.plain_rope_tables(cfg)
+        assert rope.cos.dtype == torch.float32 and tuple(rope.cos.shape) == tuple(cos.shape)
+        assert rel_err(rope.cos, cos) < 1e-6 and rel_err(rope.sin, sin) < 1e-6
+    with pytest.raises(ValueError, match="Unsupported rope_scaling_type"):
+        build_position_encoding(PartSpec("rotary", {"head_dim": 16, "rotary_dim": 16, "max_positions": 8, "theta": 1e4,
+                                                    "scaling": {"type": "bogus"}}), _ctx(torch.float32))
+
+
+@pytest.mark.parametrize("dtype,page", [(torch.float32, 8), (torch.bfloat16, 16)])
+@pytest.mark.parametrize("window", [0, 13])
+def test_attention_part_alone_in_portions(dtype, page, window):
+    """The mixer alone: a sequence fed in portions through the paged cache equals the plain
+    attention over the whole sequence; with a window, pages the window has passed are given back."""
+    from infinilm_amd.parts.registry import build_mixer
+    from infinilm_amd.config import PartSpec
+
+    H, nh, nkv, d, n = 40, 6, 2, 16, 75
+    rope_cfg = {"hidden_size": d, "num_attention_heads": 1, "rope_theta": 999.0, "max_position_embeddings": 128}
+    pos = PartSpec("rotary", {"head_dim": d, "rotary_dim": d, "max_positions": 128, "theta": 999.0, "scaling": None})
+    att = build_mixer(PartSpec("gqa_attention", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d,
+                                                 "qkv_bias": True, "out_bias": False, "scale": 0.3, "window": window,
+                                                 "position": pos}), _ctx(dtype))
+    W = _fill(att, 3)
+    hz = _Harness([att.cache_need()], dtype, page_size=page, num_pages=12)
+    x = (torch.randn(n, H) * 0.8).to(dtype)
+    outs, i = [], 0
+    for k in (17, 2, 1, 30, 1, 1, 23):
+        b = hz.batch([("r", k)])
+        outs.append(att.forward(x[i:i + k].to(DEV), b, hz.cache.view(0, b, True)))
+        hz.commit([("r", k)])
+        i += k
+    got = torch.cat(outs)
+    # plain: projections, rotation, windowed causal attention, output projection
+    xd = x.to(F64)
+    cos, sin = P.plain_rope_tables(rope_cfg)
+    q = P.plain_linear(xd, W["q_proj.weight"], W["q_proj.bias"]).view(n, nh, d)
+    k_ = P.plain_linear(xd, W["k_proj.weight"], W["k_proj.bias"]).view(n, nkv, d)
+    v = P.plain_linear(xd, W["v_proj.weight"], W["v_proj.bias"]).view(n, nkv, d)
+    p = torch.arange(n)
+    o = P.plain_attention(P.plain_apply_rope(q, p, cos, sin, d), P.plain_apply_rope(k_, p, cos, sin, d), v, 0.3, window)
+    want = P.plain_linear(o.reshape(n, nh * d), W["o_proj.weight"])
+    assert rel_err(got, want) < (5e-6 if dtype == torch.float32 else 2e-2)
+    table = hz.cache.table("r", 0)
+    if window:
+        first = (n - window + 1) // page
+        assert all(t == -1 for t in table[:first]) and all(t >= 0 for t in table[first:])
+        assert hz.cache.free_pages() == 12 - (len(table) - first)
+    else:
+        assert all(t >= 0 for t in table)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    from infinilm_amd.parts.registry import build_feed_forward
+    from infinilm_amd.config import PartSpec
+
+    ffn = build_feed_forward(PartSpec("swiglu", {"hidden_size": 80, "intermediate_size": 200, "bias": True}), _ctx(dtype))
+    W = _fill(ffn, 5)
+    for rows in (3, 70):   # the few-rows and the many-rows products
+        x = torch.randn(rows, 80).to(dtype)
+        got = ffn.forward(x.to(DEV), None)
+        want = P.plain_mlp(x.to(F64), W["gate_proj.weight"], W["up_proj.weight"], W["down_proj.weight"], 1.0,
+                           W["gate_proj.bias"], W["up_proj.bias"], W["down_proj.bias"])
+        assert rel_err(got, want) < (5e-6 if dtype == torch.float32 else 2e-2)
+
+
+# ------------------------------------------------------------------------------------------------
+# a toy architecture, defined and registered here
+# ------------------------------------------------------------------------------------------------
+def _register_toy():
+    from infinilm_amd.cache import FixedState
+    from infinilm_amd.config import HeadSpec, LayerRun, LayerSpec, ModelSpec, PartSpec, register_architecture
+    from infinilm_amd.parts import Mixer, Param, register_mixer
+
+    @register_mixer("toy_decay")
+    class ToyDecayMixer(Mixer):
+        """s_t = decay * s_{t-1} + x_t Wi^T (one state row per request), y_t = s_t Wo^T.
+        Plain tensor ops stand in for kernels: it is a toy that shows the interfaces."""
+
+        def __init__(self, hidden_size, state_size, decay, ctx):
+            self.decay = float(decay)
+            self.state_size = int(state_size)
+            self.wi = torch.empty((state_size, hidden_size), dtype=ctx.dtype, device=ctx.device)
+            self.wo = torch.empty((hidden_size, state_size), dtype=ctx.dtype, device=ctx.device)
+
+        def named_parameters(self):
+            return {"in_proj.weight": Param(self.wi), "out_proj.weight": Param(self.wo)}
+
+        def cache_need(self):
+            return FixedState((self.state_size,), torch.float32)
+
+        def forward(self, x, batch, view):
+            u = x.float() @ self.wi.float().t()
+            out = torch.empty_like(u)
+            off = batch.h_seg_offsets
+            for i in range(batch.R):
+                s = view.pool[int(batch.h_state_in[i])].clone()
+                for t in range(int(off[i]), int(off[i + 1])):
+                    s = self.decay * s + u[t]
+                    out[t] = s
+                view.pool[int(batch.h_state_out[i])] = s
+            return (out @ self.wo.float().t()).to(x.dtype)
+
+    def config_from_dict(raw):
+        return dict(raw)
+
+    def build_spec(cfg):
+        H, d = cfg["hidden_size"], cfg["head_dim"]
+        norm = PartSpec("rmsnorm", {"size": H, "eps": cfg["eps"]})
+        pos = PartSpec("rotary", {"head_dim": d, "rotary_dim": d, "max_positions": cfg["max_positions"], "theta": 1e4,
+                                  "scaling": None})
+        att = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": cfg["heads"], "num_kv_heads": cfg["kv_heads"],
+                                         "head_dim": d, "qkv_bias": False, "out_bias": False, "scale": d ** -0.5,
+                                         "window": 0, "position": pos})
+        toy = PartSpec("toy_decay", {"hidden_size": H, "state_size": cfg["state_size"], "decay": cfg["decay"]})
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": cfg["intermediate_size"], "bias": False})
+        names = {"norm1": "ln1", "mixer": "mix", "norm2": "ln2", "ffn": "ffn"}
+        mixers = [att, toy, att]
+        layers = [LayerSpec(f"blocks.{i}", "pre_norm", {"norm1": norm, "mixer": m, "norm2": norm, "ffn": ffn}, names, 0.5)
+                  for i, m in enumerate(mixers)]
+        # layer 1 (the toy mixer) runs twice with states of its own; layer 2 reads layer 0's keys and values
+        order = [LayerRun(0, 0), LayerRun(1, 1), LayerRun(2, 0, writes_cache=False), LayerRun(1, 2)]
+        return ModelSpec("ToyForCausalLM", cfg["vocab_size"], H, cfg["max_positions"], "emb", 1.0, layers, order, norm,
+                         "ln_f", HeadSpec("head", 1.0, True))
+
+    register_architecture(["ToyForCausalLM"], config_from_dict, build_spec)
+
+
+def _toy_plain(cfg, W, ids):
+    """The toy model, whole sequence, in float64."""
+    W = {k: v.to(F64) for k, v in W.items()}
+    n, H, d, nh, nkv = len(ids), cfg["hidden_size"], cfg["head_dim"], cfg["heads"], cfg["kv_heads"]
+    cos, sin = P.plain_rope_tables({"hidden_size": d, "num_attention_heads": 1, "max_position_embeddings": cfg["max_positions"]})
+    pos = torch.arange(n)
+    x = W["emb.weight"][torch.tensor(ids)]
+    kv0 = None
+
+    def toy(h, p):
+        u = h @ W[p + "in_proj.weight"].T
+        s = torch.zeros(cfg["state_size"], dtype=F64)
+        out = []
+        for t in range(n):
+            s = cfg["decay"] * s + u[t]
+            out.append(s)
+        return torch.stack(out) @ W[p + "out_proj.weight"].T
+
+    for layer, reads_layer0 in ((0, False), (1, None), (2, True), (1, None)):
+        p = f"blocks.{layer}."
+        h = P.plain_rmsnorm(x, W[p + "ln1.weight"], cfg["eps"])
+        if reads_layer0 is None:
+            y = toy(h, p + "mix.")
+        else:
+            q = P.plain_apply_rope(P.plain_linear(h, W[p + "mix.q_proj.weight"]).view(n, nh, d), pos, cos, sin, d)
+            if not reads_layer0:
+                k = P.plain_apply_rope(P.plain_linear(h, W[p + "mix.k_proj.weight"]).view(n, nkv, d), pos, cos, sin, d)
+                v = P.plain_linear(h, W[p + "mix.v_proj.weight"]).view(n, nkv, d)
+                kv0 = (k, v)
+            o = P.plain_attention(q, kv0[0], kv0[1], d ** -0.5).reshape(n, nh * d)
+            y = P.plain_linear(o, W[p + "mix.o_proj.weight"])
+        x = x + 0.5 * y
+        h = P.plain_rmsnorm(x, W[p + "ln2.weight"], cfg["eps"])
+        x = x + 0.5 * P.plain_mlp(h, W[p + "ffn.gate_proj.weight"], W[p + "ffn.up_proj.weight"], W[p + "ffn.down_proj.weight"], 1.0)
+    return P.plain_linear(P.plain_rmsnorm(x, W["ln_f.weight"], cfg["eps"]), W["emb.weight"])
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
+    from safetensors.torch import save_file
+    from infinilm_amd.engine.loading import build_model
+    from helpers import Driver
+
+    _register_toy()
+    cfg = {"architectures": ["ToyForCausalLM"], "torch_dtype": "float32", "vocab_size": 97, "hidden_size": 48,
+           "head_dim": 16, "heads": 4, "kv_heads": 2, "intermediate_size": 72, "state_size": 24, "decay": 0.9,
+           "eps": 1e-5, "max_positions": 256}
+    d = str(tmp_path / "toy")
+    os.makedirs(d)
+    json.dump(cfg, open(os.path.join(d, "config.json"), "w"))
+    meta = build_model(cfg, "float32", "meta")
+    names = meta.named_parameters()
+    assert "blocks.1.mix.in_proj.weight" in names and "blocks.2.mix.q_proj.weight" in names
+    g = torch.Generator().manual_seed(4)
+    W = {}
+    for name, p in sorted(names.items()):
+        if name == "head.weight":
+            continue   # tied to the embedding
+        t = torch.randn(tuple(p.tensor.shape), generator=g) * (0.3 if len(p.tensor.shape) == 2 else 0.1)
+        W[name] = (t + 1.0) if t.dim() == 1 else t
+    save_file(W, os.path.join(d, "model.safetensors"), metadata={"format": "pt"})
+
+    drv = Driver(d, "float32", num_pages=24, page_size=8, max_requests=3)
+    from infinilm_amd.cache import FixedState, PagedKV
+    needs = drv.model.cache_needs
+    assert isinstance(needs[0], PagedKV) and isinstance(needs[1], FixedState) and isinstance(needs[2], FixedState)
+    g2 = torch.Generator().manual_seed(9)
+    seqs = {r: torch.randint(0, 97, (n,), generator=g2).tolist() for r, n in (("a", 50), ("b", 21), ("c", 33))}
+    # a in portions, b whole beside a's portions, then c in a slot that b has given back
+    drv.step([("a", seqs["a"][:20])])
+    drv.step([("a", seqs["a"][20:22]), ("b", seqs["b"])], end=["b"])
+    drv.step([("a", seqs["a"][22:23]), ("c", seqs["c"][:5])])
+    drv.step([("c", seqs["c"][5:]), ("a", seqs["a"][23:])], end=["a", "c"])
+    for r, ids in seqs.items():
+        err = rel_err(drv.request_logits(r, len(ids)), _toy_plain(cfg, W, ids))
+        assert err < 1e-4, f"request {r}: error {err:.3e}"
+    assert drv.runner.cache.free_pages() == 24
