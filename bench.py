@@ -56,6 +56,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step eagerly")
+    ap.add_argument("--prefill-only", action="store_true", help="only the prefill measurement (for profiling)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -129,6 +130,29 @@ def main() -> int:
         step_bytes = layer_weight_bytes + head_bytes + batch * H * esize + kv_bytes
         return {"tok_s": batch * steps / dt, "ms": ms, "bytes": step_bytes, "gbs": step_bytes / (dt / steps) / 1e9}
 
+    def prefill():
+        # one prompt of T tokens in one step, logits at its last place
+        T = args.prefill_tokens
+        prompt = torch.randint(0, V, (T,), generator=gen).tolist()
+        times = []
+        for i in range(3):
+            rid = f"p{i}"
+            cache.admit(rid)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            logits = runner.step([StepEntry(rid, prompt, [T - 1])])
+            sampler.sample(logits, [(greedy, 0, 0)])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            cache.release(rid)
+        pt = min(times[1:])
+        mat_params = sum(p.tensor.numel() for n, p in model.named_parameters().items() if ".layers." in n and p.tensor.dim() == 2)
+        flops = 2.0 * T * mat_params + 4.0 * T * T / 2.0 * 32 * 128 * L + 2.0 * V * H
+        return {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3), "frac": round(flops / pt / FLOP_PEAK[dkey], 4)}
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": prefill()}))
+        return 0
     main_pt = decode(args.batch, args.steps, args.warmup)
     record = {
         "metric": "decode tokens/s, MiniCPM4-8B shape, batch %d, context %d" % (args.batch, args.context),
@@ -147,25 +171,7 @@ def main() -> int:
         k = max(8, args.steps // 2)
         record["points"] = {"decode_b1": round(decode(1, k, args.warmup)["tok_s"], 2),
                             "decode_b64": round(decode(64, k, args.warmup)["tok_s"], 2)}
-        # prefill: one prompt of T tokens in one step, logits at its last place
-        T = args.prefill_tokens
-        prompt = torch.randint(0, V, (T,), generator=gen).tolist()
-        times = []
-        for i in range(3):
-            rid = f"p{i}"
-            cache.admit(rid)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            logits = runner.step([StepEntry(rid, prompt, [T - 1])])
-            sampler.sample(logits, [(greedy, 0, 0)])
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t0)
-            cache.release(rid)
-        pt = min(times[1:])
-        mat_params = sum(p.tensor.numel() for n, p in model.named_parameters().items() if ".layers." in n and p.tensor.dim() == 2)
-        flops = 2.0 * T * mat_params + 4.0 * T * T / 2.0 * 32 * 128 * L + 2.0 * V * H
-        record["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                             "frac": round(flops / pt / FLOP_PEAK[dkey], 4)}
+        record["prefill"] = prefill()
     print(json.dumps(record))
     return 0
 

@@ -168,11 +168,14 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     if a.dtype == BF16 and not FORCE_BASIC:
         aligned = K % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 \
             and w.data_ptr() % 16 == 0
-        if M <= 64 and aligned:
+        library_ok = bias is None and alpha == 1.0 and out_dtype == BF16 and USE_LIBRARY_GEMM
+        # measured at the 8B shapes: the few-rows kernel beats the vendor library up to 16 rows and
+        # loses to it above (its X fragments are re-read from L2 for every 16 rows of W)
+        if M <= 64 and aligned and not (M > 16 and library_ok):
             _run("ilm_gemm_skinny", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
                  w.stride(0), out.stride(0), float(alpha), _DT[out_dtype], SKINNY_VARIANT, _stream())
             return out
-        if M > 64 and bias is None and alpha == 1.0 and out_dtype == BF16 and USE_LIBRARY_GEMM:
+        if M > 16 and library_ok:
             # large products go to the vendor library, as the reference's linear layers do
             # (csrc/layers/quantization/none_quantization.cpp:26-46 calls its library's linear)
             torch.matmul(a, w.t(), out=out)

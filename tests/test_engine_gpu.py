@@ -101,6 +101,32 @@ def test_graph_replays_equal_eager_steps(models):
     assert len(graph._graphs) >= 2   # the context outgrew the first graph's block-table width
 
 
+def test_graph_with_many_requests_replays_like_eager(models):
+    """More than 16 decoded tokens a step: the projections go to the vendor library inside the
+    captured graph; replays must still equal eager steps, several times over."""
+    from infinilm_amd.engine.loading import load_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+
+    cfg, d, W = models[("A", "bfloat16")]
+    model = load_model(d, "bfloat16", "cuda:0")
+    n = 20
+    eager = make_runner(model, num_pages=64, page_size=16, max_requests=n)
+    graph = make_runner(model, num_pages=64, page_size=16, max_requests=n, enable_graph=True)
+    prompts = {f"r{i}": random_tokens(cfg, 3 + i, 50 + i) for i in range(n)}
+    for r in (eager, graph):
+        for rid, p in prompts.items():
+            r.cache.admit(rid)
+        r.step([StepEntry(rid, p, []) for rid, p in prompts.items()])
+    nxt = {rid: 11 + i for i, rid in enumerate(prompts)}
+    for step in range(12):
+        entries = [StepEntry(rid, [t], [0]) for rid, t in nxt.items()]
+        le = eager.step(entries).clone()
+        torch.cuda.synchronize()
+        lg = graph.step(entries)
+        assert rel_err(lg, le) < 1e-6, f"replay {step} differs from the eager step"
+        nxt = {rid: int(torch.argmax(le[i])) for i, rid in enumerate(prompts)}
+
+
 def test_seeded_sampling_is_reproducible_and_independent_of_the_batch(models):
     from infinilm_amd import LLM, SamplingParams
 
