@@ -1,6 +1,9 @@
 // Paged attention on the matrix cores (bfloat16 in, float softmax and accumulation).
 //
-// Same contract as attn_basic.hip.  A workgroup of 4 waves serves one token and one group of up to
+// Same contract as attn_basic.hip.  Two kernels: single tokens (decoding) over key chunks, below,
+// and tiles of consecutive tokens of one request (portions of prompts), further down.
+//
+// Single tokens: `rows` (optional) lists the token rows to serve.  A workgroup of 4 waves serves one token and one group of up to
 // 16 query heads that share a KV head, over one chunk of ATT_CHUNK keys; each wave takes a quarter
 // of the chunk, the four partial results are merged through LDS.  Chunks are aligned to absolute
 // key index, so what is summed in which order depends on (request, position) alone.  With more
@@ -41,13 +44,13 @@ __global__ void __launch_bounds__(ATT_WAVES * 64)
 attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
                  const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                  const int* __restrict__ block_tables, const int* __restrict__ seg,
-                 const int* __restrict__ pos, int nh, int nkv, int page, int max_blocks, int q_stride,
-                 int out_stride, float scale_log2e, int window, int nsplit) {
+                 const int* __restrict__ pos, const int* __restrict__ rows, int nh, int nkv, int page,
+                 int max_blocks, int q_stride, int out_stride, float scale_log2e, int window, int nsplit) {
     constexpr int D = D16 * 16;
     constexpr int KS = (D + 31) / 32;
     __shared__ float sm_acc[ATT_WAVES][D16][64][4];
     __shared__ float sm_ml[ATT_WAVES][16][2];
-    const int t = blockIdx.x;
+    const int t = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
     const int G = nh / nkv;
     const int HG = (G + 15) / 16;
     const int kvh = blockIdx.y / HG, hg = blockIdx.y % HG;
@@ -229,9 +232,11 @@ attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __re
 // One wave per (token, head); lanes first share the chunks' (m, l), then each sums its dims.
 __global__ void __launch_bounds__(64)
 attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
-                  const int* __restrict__ pos, int nh, int D, int out_stride, int window, int nsplit) {
+                  const int* __restrict__ pos, const int* __restrict__ rows, int nh, int D, int out_stride,
+                  int window, int nsplit) {
     __shared__ float wsm[64];
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int t = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
+    const int h = blockIdx.y, lane = threadIdx.x;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int s_lo = lo / ATT_CHUNK, s_hi = p / ATT_CHUNK;
@@ -271,12 +276,250 @@ attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, cons
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Tiles of up to ATT_TT consecutive tokens of one request (portions of prompts): the 4 waves of a
+// workgroup take 2 tokens each and share every 32-key tile of K and V through LDS (double
+// buffered), so a tile is read from the cache once per 8 tokens x 16 heads.  No key chunks and no
+// workspace: one workgroup walks all keys its tokens see, in ascending order of absolute key
+// index, 32 at a time.
+// ------------------------------------------------------------------------------------------------
+#define ATT_TT 8
+#define ATT_NT 2
+
+template <int D16>
+__global__ void __launch_bounds__(256)
+attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ kc,
+                 const bf16* __restrict__ vc, const int* __restrict__ block_tables, const int* __restrict__ seg,
+                 const int* __restrict__ pos, const int* __restrict__ tiles, int nh, int nkv, int page,
+                 int max_blocks, int q_stride, int out_stride, float scale_log2e, int window) {
+    constexpr int D = D16 * 16;
+    constexpr int KS = (D + 31) / 32;
+    constexpr int KROW = D + 8;    // padded rows: conflict-free 16-byte reads of 16 rows
+    constexpr int VROW = 32 + 8;
+    __shared__ __attribute__((aligned(16))) bf16 Ks[2][32][KROW];
+    __shared__ __attribute__((aligned(16))) bf16 Vs[2][D][VROW];
+    const int t0 = tiles[2 * blockIdx.x], ntok = tiles[2 * blockIdx.x + 1];
+    const int G = nh / nkv;
+    const int HG = (G + 15) / 16;
+    const int kvh = blockIdx.y / HG, hg = blockIdx.y % HG;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, qg = lane >> 4;
+    const int hcol = hg * 16 + r;
+    const bool head_ok = hcol < G;
+    const int head = kvh * G + (head_ok ? hcol : G - 1);
+    const int p_first = pos[t0], p_last = p_first + ntok - 1;
+    const int lo_first = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+    const int* bt = block_tables + (size_t)seg[t0] * max_blocks;
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+
+    // this wave's tokens
+    int tok[ATT_NT], pj[ATT_NT], loj[ATT_NT];
+    bool tok_ok[ATT_NT];
+    uint4 qf[ATT_NT][KS];
+#pragma unroll
+    for (int j = 0; j < ATT_NT; ++j) {
+        const int i = wave * ATT_NT + j;
+        tok_ok[j] = i < ntok;
+        tok[j] = t0 + (tok_ok[j] ? i : ntok - 1);
+        pj[j] = p_first + (tok_ok[j] ? i : ntok - 1);
+        loj[j] = (window > 0 && pj[j] - window + 1 > 0) ? pj[j] - window + 1 : 0;
+        const bf16* qrow = q + (size_t)tok[j] * q_stride + (size_t)head * D;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int dofs = ks * 32 + qg * 8;
+            const uint4 v = *reinterpret_cast<const uint4*>(qrow + (dofs < D ? dofs : 0));
+            qf[j][ks] = dofs < D ? v : zero4;
+        }
+    }
+    f32x4 acc[ATT_NT][D16];
+    float m[ATT_NT], lsum[ATT_NT];
+#pragma unroll
+    for (int j = 0; j < ATT_NT; ++j) {
+        m[j] = NEG_BIG;
+        lsum[j] = 0.f;
+#pragma unroll
+        for (int db = 0; db < D16; ++db) acc[j][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // cooperative copy of one 32-key tile: K rows [key][d], V rows [d][key]
+    constexpr int KPIECES = 32 * (D / 8);   // 16-byte pieces
+    constexpr int VPIECES = D * 4;
+    constexpr int KPER = (KPIECES + 255) / 256, VPER = (VPIECES + 255) / 256;
+    static_assert(KPER <= 2 && VPER <= 2, "a tile is at most two 16-byte pieces a thread");
+    auto fetch_k = [&](int kb, int i) -> uint4 {
+        const int pc = tid + i * 256;
+        const int row = (pc < KPIECES ? pc : 0) / (D / 8), col = (pc < KPIECES ? pc : 0) % (D / 8);
+        int key = kb + row;
+        key = key < lo_first ? lo_first : (key > p_last ? p_last : key);   // a page that exists
+        const int pg = bt[key / page];
+        return *reinterpret_cast<const uint4*>(kc + (((size_t)pg * nkv + kvh) * page + (key % page)) * D + col * 8);
+    };
+    auto fetch_v = [&](int kb, int i) -> uint4 {
+        const int pc = tid + i * 256;
+        const int drow = (pc < VPIECES ? pc : 0) >> 2, kgrp = (pc < VPIECES ? pc : 0) & 3;
+        int key0 = kb + kgrp * 8;
+        if (key0 > p_last || key0 + 8 <= lo_first) key0 = lo_first & ~7;   // masked later; any valid group
+        const int pg = bt[key0 / page];
+        return *reinterpret_cast<const uint4*>(vc + (((size_t)pg * nkv + kvh) * D + drow) * page + (key0 % page));
+    };
+    auto stash_k = [&](int buf, int i, uint4 v) {
+        const int pc = tid + i * 256;
+        if (pc < KPIECES) *reinterpret_cast<uint4*>(&Ks[buf][pc / (D / 8)][(pc % (D / 8)) * 8]) = v;
+    };
+    auto stash_v = [&](int buf, int i, uint4 v) {
+        const int pc = tid + i * 256;
+        if (pc < VPIECES) *reinterpret_cast<uint4*>(&Vs[buf][pc >> 2][(pc & 3) * 8]) = v;
+    };
+    uint4 k0 = zero4, k1 = zero4, v0 = zero4, v1 = zero4;
+#define ATT_FETCH(kb_)                          \
+    k0 = fetch_k(kb_, 0);                       \
+    if (KPER > 1) k1 = fetch_k(kb_, 1);         \
+    v0 = fetch_v(kb_, 0);                       \
+    if (VPER > 1) v1 = fetch_v(kb_, 1);
+#define ATT_STASH(buf_)                         \
+    stash_k(buf_, 0, k0);                       \
+    if (KPER > 1) stash_k(buf_, 1, k1);         \
+    stash_v(buf_, 0, v0);                       \
+    if (VPER > 1) stash_v(buf_, 1, v1);
+
+    const int kb0 = lo_first & ~31;
+    ATT_FETCH(kb0)
+    ATT_STASH(0)
+    __syncthreads();
+    int buf = 0;
+    for (int kb = kb0; kb <= p_last; kb += 32, buf ^= 1) {
+        const bool more = kb + 32 <= p_last;
+        if (more) { ATT_FETCH(kb + 32) }
+        // ---- this wave's tokens against the tile in Ks[buf], Vs[buf]
+        const bool any = kb <= pj[ATT_NT - 1] && kb + 32 > loj[0];   // wave-uniform
+        if (any) {
+            f32x4 s[ATT_NT][2];
+#pragma unroll
+            for (int tau = 0; tau < 2; ++tau) {
+                const int row = (r >> 2) * 8 + tau * 4 + (r & 3);
+                uint4 kf[KS];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const int dofs = ks * 32 + qg * 8;
+                    kf[ks] = dofs < D ? *reinterpret_cast<const uint4*>(&Ks[buf][row][dofs]) : zero4;
+                }
+#pragma unroll
+                for (int j = 0; j < ATT_NT; ++j) {
+                    s[j][tau] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) s[j][tau] = mfma16(kf[ks], qf[j][ks], s[j][tau]);
+                }
+            }
+            uint4 pf[ATT_NT];
+            float corr[ATT_NT];
+#pragma unroll
+            for (int j = 0; j < ATT_NT; ++j) {
+                float sv[8];
+                float mx = NEG_BIG;
+#pragma unroll
+                for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int key = kb + qg * 8 + tau * 4 + e;
+                        const bool ok = key >= loj[j] && key <= pj[j];
+                        const float v = ok ? s[j][tau][e] * scale_log2e : NEG_BIG;
+                        sv[tau * 4 + e] = v;
+                        mx = fmaxf(mx, v);
+                    }
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                const float m_new = fmaxf(m[j], mx);
+                corr[j] = __builtin_amdgcn_exp2f(m[j] - m_new);
+                float pe[8];
+                float rs = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    pe[i] = (sv[i] > 0.5f * NEG_BIG) ? __builtin_amdgcn_exp2f(sv[i] - m_new) : 0.f;
+                    rs += pe[i];
+                }
+                rs += __shfl_xor(rs, 16, 64);
+                rs += __shfl_xor(rs, 32, 64);
+                lsum[j] = lsum[j] * corr[j] + rs;
+                m[j] = m_new;
+                pf[j].x = pack_bf16x2(pe[0], pe[1]);
+                pf[j].y = pack_bf16x2(pe[2], pe[3]);
+                pf[j].z = pack_bf16x2(pe[4], pe[5]);
+                pf[j].w = pack_bf16x2(pe[6], pe[7]);
+            }
+            const int key0 = kb + qg * 8;
+            const bool vok = key0 <= p_last && key0 + 8 > lo_first;   // else the tile holds another group's values
+#pragma unroll
+            for (int db = 0; db < D16; ++db) {
+                const uint4 v = *reinterpret_cast<const uint4*>(&Vs[buf][db * 16 + r][qg * 8]);
+                const uint4 vf = vok ? v : zero4;
+#pragma unroll
+                for (int j = 0; j < ATT_NT; ++j) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[j][db][e] *= corr[j];
+                    acc[j][db] = mfma16(vf, pf[j], acc[j][db]);
+                }
+            }
+        }
+        if (more) { ATT_STASH(buf ^ 1) }
+        __syncthreads();
+    }
+    if (!head_ok) return;
+#pragma unroll
+    for (int j = 0; j < ATT_NT; ++j) {
+        if (!tok_ok[j]) continue;
+        const float inv = 1.0f / lsum[j];
+        bf16* orow = out + (size_t)tok[j] * out_stride + (size_t)head * D;
+#pragma unroll
+        for (int db = 0; db < D16; ++db) {
+            uint2 w;
+            w.x = pack_bf16x2(acc[j][db][0] * inv, acc[j][db][1] * inv);
+            w.y = pack_bf16x2(acc[j][db][2] * inv, acc[j][db][3] * inv);
+            *reinterpret_cast<uint2*>(orow + db * 16 + qg * 4) = w;
+        }
+    }
+}
+
+#undef ATT_FETCH
+#undef ATT_STASH
+
+extern "C" int ilm_attn_tile_tokens() { return ATT_TT; }
+
+extern "C" int ilm_attn_tile(void* out, const void* q, const void* kc, const void* vc, const void* block_tables,
+                             const void* seg, const void* pos, const void* tiles, int n_tiles, int nh, int nkv,
+                             int d, int page, int max_blocks, int q_stride, int out_stride, float scale,
+                             int window, hipStream_t stream) {
+    ILM_REQUIRE(n_tiles > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_tile: bad sizes");
+    ILM_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attn_tile: head size %d is not a multiple of 16 up to 128", d);
+    ILM_REQUIRE(page % 16 == 0 && page > 0, "attn_tile: page size %d is not a multiple of 16", page);
+    ILM_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0 && ((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 7) == 0,
+                "attn_tile: q and out rows must be 16-byte / 8-byte aligned");
+    const int G = nh / nkv, HG = (G + 15) / 16;
+    ILM_REQUIRE(nkv * HG <= 65535, "attn_tile: grid too large");
+    dim3 grid(n_tiles, nkv * HG);
+    const float sl2 = scale * 1.4426950408889634f;
+#define AT_CASE(D16)                                                                                            \
+    case D16:                                                                                                   \
+        attn_tile_kernel<D16><<<grid, 256, 0, stream>>>((bf16*)out, (const bf16*)q, (const bf16*)kc, (const bf16*)vc, \
+                                                        (const int*)block_tables, (const int*)seg, (const int*)pos, \
+                                                        (const int*)tiles, nh, nkv, page, max_blocks, q_stride, \
+                                                        out_stride, sl2, window);                               \
+        break
+    switch (d / 16) {
+        AT_CASE(1); AT_CASE(2); AT_CASE(3); AT_CASE(4); AT_CASE(5); AT_CASE(6); AT_CASE(7); AT_CASE(8);
+        default: ILM_REQUIRE(false, "attn_tile: head size %d", d);
+    }
+#undef AT_CASE
+    ILM_LAUNCH_CHECK("attn_tile");
+    return 0;
+}
+
+
 extern "C" int ilm_attn_mfma_chunk() { return ATT_CHUNK; }
 
 extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q, const void* kc,
                              const void* vc, const void* block_tables, const void* seg, const void* pos,
-                             int T_, int nh, int nkv, int d, int page, int max_blocks, int q_stride,
-                             int out_stride, float scale, int window, int nsplit, hipStream_t stream) {
+                             const void* rows, int T_, int nh, int nkv, int d, int page, int max_blocks,
+                             int q_stride, int out_stride, float scale, int window, int nsplit,
+                             hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_mfma: bad head counts nh=%d nkv=%d", nh, nkv);
     ILM_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attn_mfma: head size %d is not a multiple of 16 up to 128", d);
     ILM_REQUIRE(page % 16 == 0 && page > 0, "attn_mfma: page size %d is not a multiple of 16", page);
@@ -291,8 +534,8 @@ extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q
     case D16:                                                                                                  \
         attn_mfma_kernel<D16><<<grid, ATT_WAVES * 64, 0, stream>>>(                                            \
             (bf16*)out, (float*)ws_acc, (float*)ws_ml, (const bf16*)q, (const bf16*)kc, (const bf16*)vc,      \
-            (const int*)block_tables, (const int*)seg, (const int*)pos, nh, nkv, page, max_blocks, q_stride,  \
-            out_stride, sl2, window, nsplit);                                                                  \
+            (const int*)block_tables, (const int*)seg, (const int*)pos, (const int*)rows, nh, nkv, page,      \
+            max_blocks, q_stride, out_stride, sl2, window, nsplit);                                            \
         break
     switch (d / 16) {
         AM_CASE(1); AM_CASE(2); AM_CASE(3); AM_CASE(4); AM_CASE(5); AM_CASE(6); AM_CASE(7); AM_CASE(8);
@@ -303,7 +546,7 @@ extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q
     if (nsplit > 1) {
         dim3 g2(T_, nh);
         attn_merge_kernel<<<g2, 64, 0, stream>>>((bf16*)out, (const float*)ws_acc, (const float*)ws_ml, (const int*)pos,
-                                                 nh, d, out_stride, window, nsplit);
+                                                 (const int*)rows, nh, d, out_stride, window, nsplit);
         ILM_LAUNCH_CHECK("attn_merge");
     }
     return 0;

@@ -43,6 +43,8 @@ class StepBatch:
         self.want_rows = None           # [num_wanted] rows of the flattened batch
         self.state_in = None            # [R] state row read at the start (0 = zeros)
         self.state_out = None           # [R] state row written at the end
+        self.att_tiles = None           # [n, 2] (first row, count): runs of <= 8 consecutive tokens of one request
+        self.att_single_rows = None     # rows of requests that bring one token (None: no run of 2 or more exists)
         self.block_tables: List = []    # per group [R, max_blocks], -1 padded
         self.slots: List = []           # per group [T] slot of each new token
         self.num_wanted = 0
@@ -131,9 +133,24 @@ class StepRunner:
         max_blocks = [max(1, min_blocks, max(len(cache.table(e.req_id, g)) for e in entries)) for g in range(G)]
         n_want = sum(len(e.want) for e in entries)
 
+        # attention work lists: runs of up to TILE consecutive tokens of a request, and single tokens
+        TILE = 8
+        tiles: List[int] = []
+        singles: List[int] = []
+        for i in range(R):
+            a, n = int(offsets[i]), int(lens[i])
+            if n == 1:
+                singles.append(a)
+            else:
+                for k in range(0, n, TILE):
+                    tiles += [a + k, min(TILE, n - k)]
+        if not tiles:
+            singles = []   # every token is single: the kernels take all rows
+
         # layout of the one int32 buffer
         sizes = [("token_ids", T), ("positions", T), ("seg_of_token", T), ("seg_offsets", R + 1), ("start_pos", R),
-                 ("total_lens", R), ("want_rows", n_want), ("state_in", R), ("state_out", R)]
+                 ("total_lens", R), ("want_rows", n_want), ("state_in", R), ("state_out", R),
+                 ("att_tiles", len(tiles)), ("att_singles", len(singles))]
         for g in range(G):
             sizes.append((f"slots{g}", T))
             sizes.append((f"bt{g}", R * max_blocks[g]))
@@ -165,6 +182,8 @@ class StepRunner:
             for x in e.want:
                 w[k] = offsets[i] + x
                 k += 1
+        seg("att_tiles")[:] = tiles
+        seg("att_singles")[:] = singles
         sin, sout = seg("state_in"), seg("state_out")
         for i, e in enumerate(entries):
             sin[i], sout[i] = cache.state_rows(e.req_id)
@@ -201,6 +220,9 @@ class StepRunner:
         b.token_ids, b.positions, b.seg_of_token = dseg("token_ids"), dseg("positions"), dseg("seg_of_token")
         b.seg_offsets, b.start_pos, b.total_lens = dseg("seg_offsets"), dseg("start_pos"), dseg("total_lens")
         b.want_rows, b.state_in, b.state_out = dseg("want_rows"), dseg("state_in"), dseg("state_out")
+        if tiles:
+            b.att_tiles = dseg("att_tiles").view(-1, 2)
+            b.att_single_rows = dseg("att_singles") if singles else None
         b.block_tables = [dseg(f"bt{g}").view(R, max_blocks[g]) for g in range(G)]
         b.slots = [dseg(f"slots{g}") for g in range(G)]
         b.num_wanted = n_want

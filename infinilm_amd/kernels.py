@@ -17,6 +17,7 @@ from .csrc import lib as _libmod
 F32 = torch.float32
 BF16 = torch.bfloat16
 _DT = {torch.float32: 0, torch.bfloat16: 1}
+ATT_TILE_TOKENS = 8  # tokens per tile of the prompt-portion attention kernel (ilm_attn_tile_tokens())
 ATT_CHUNK = 256  # keys per chunk of the matrix-core attention kernel (ilm_attn_mfma_chunk())
 # INFINILM_AMD_BASIC=1 runs the plain kernels everywhere (for telling a kernel's fault from the engine's)
 FORCE_BASIC = os.environ.get("INFINILM_AMD_BASIC", "0") == "1"
@@ -187,13 +188,16 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int,
-                    scale: float, window: int = 0, max_total_len: Optional[int] = None) -> torch.Tensor:
+                    scale: float, window: int = 0, max_total_len: Optional[int] = None,
+                    tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of every token over its request's cached keys up to its own position.
 
     q: rows of T tokens in which head h lies at [h*d, (h+1)*d) (a view into the fused projection is
     fine); caches as the cache manager lays them out; block_tables [R, max_blocks]; `max_total_len`: an
     upper bound of position + 1 over the batch (the matrix-core kernel sizes its key chunks by it;
-    without it the plain kernel runs).  Returns [T, nh*d]."""
+    without it the plain kernel runs).  `tiles` [n, 2] = (first row, count <= ATT_TILE_TOKENS) lists runs of
+    consecutive tokens of one request and `single_rows` the remaining rows; without them every token
+    is served on its own.  Returns [T, nh*d]."""
     _dev(q, k_cache, v_cache, block_tables, seg_of_token, positions)
     _i32(block_tables, "block_tables")
     _i32(seg_of_token, "seg_of_token")
@@ -209,14 +213,28 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     out = torch.empty((T, nh * d), dtype=q.dtype, device=q.device)
     if (q.dtype == BF16 and not FORCE_BASIC and d % 16 == 0 and d <= 128 and page % 16 == 0 and q.stride(0) % 8 == 0
             and max_total_len is not None):
+        n_single = T
+        rows = None
+        if tiles is not None and tiles.numel() > 0:
+            # portions of prompts: tiles of consecutive tokens share their keys through LDS
+            _i32(tiles, "tiles")
+            _run("ilm_attn_tile", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                 block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), tiles.data_ptr(),
+                 tiles.numel() // 2, nh, nkv, d, page, block_tables.shape[1], q.stride(0), out.stride(0), float(scale),
+                 int(window), _stream())
+            if single_rows is None or single_rows.numel() == 0:
+                return out
+            _i32(single_rows, "single_rows")
+            rows, n_single = single_rows, single_rows.numel()
         nsplit = max(1, -(-int(max_total_len) // ATT_CHUNK))
         ws_acc = ws_ml = None
         if nsplit > 1:
             ws_acc = torch.empty((T * nh * nsplit * d,), dtype=F32, device=q.device)
             ws_ml = torch.empty((T * nh * nsplit * 2,), dtype=F32, device=q.device)
         _run("ilm_attn_mfma", out.data_ptr(), _ptr(ws_acc), _ptr(ws_ml), q.data_ptr(), k_cache.data_ptr(),
-             v_cache.data_ptr(), block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d,
-             page, block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window), nsplit, _stream())
+             v_cache.data_ptr(), block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), _ptr(rows),
+             n_single, nh, nkv, d, page, block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window),
+             nsplit, _stream())
         return out
     _run("ilm_attn_basic", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
          seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d, page, block_tables.shape[1],

@@ -185,9 +185,20 @@ def _attention_case(K, dtype, nh, nkv, d, page, lens, qlens, window=0, seed=0, s
         seg += [i] * ql
         pos += list(range(n - ql, n))
     q = torch.cat(q_rows).reshape(-1, nh * d)
+    # work lists as the step function builds them: runs of up to 8 tokens of a request, and single tokens
+    tiles, singles, row = [], [], 0
+    for ql in qlens:
+        if ql == 1:
+            singles.append(row)
+        else:
+            for k in range(0, ql, 8):
+                tiles += [row + k, min(8, ql - k)]
+        row += ql
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    extra = dict(tiles=i32(tiles).view(-1, 2), single_rows=i32(singles) if singles else None) if tiles else {}
     out = K.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), torch.tensor(seg, dtype=torch.int32, device=DEV),
                             torch.tensor(pos, dtype=torch.int32, device=DEV), nh, nkv, d, 1 / math.sqrt(d), window,
-                            max_total_len=max(lens))
+                            max_total_len=max(lens), **extra)
     want = []
     for i, (n, ql) in enumerate(zip(lens, qlens)):
         full = P.plain_attention(qs[i].to(F64), ks[i].to(F64), vs[i].to(F64), 1 / math.sqrt(d), window)
