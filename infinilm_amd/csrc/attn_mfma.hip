@@ -31,8 +31,13 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 #define ATT_ITERS (ATT_WKEYS / 32)
 #define NEG_BIG (-1.0e30f)
 
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+// two floats to packed bfloat16, round to nearest even (one v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
 __device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
@@ -278,31 +283,37 @@ attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, cons
 
 // ------------------------------------------------------------------------------------------------
 // Tiles of up to ATT_TT consecutive tokens of one request (portions of prompts): the 4 waves of a
-// workgroup take 2 tokens each and share every 32-key tile of K and V through LDS (double
-// buffered), so a tile is read from the cache once per 8 tokens x 16 heads.  No key chunks and no
+// workgroup take 2 tokens each and share every 64-key tile of K and V through LDS (the next tile is
+// already on its way into registers), so a tile is read from the cache once per 8 tokens x 16 heads.  No key chunks and no
 // workspace: one workgroup walks all keys its tokens see, in ascending order of absolute key
 // index, 32 at a time.
 // ------------------------------------------------------------------------------------------------
 #define ATT_TT 8
 #define ATT_NT 2
+#define ATT_TK 64        // keys per tile
+#define ATT_BT_LDS 2048  // block-table entries kept in LDS
 
-template <int D16>
-__global__ void __launch_bounds__(256)
+template <int D16, bool PAGE64>
+__global__ void __launch_bounds__(256, 2)
 attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ kc,
                  const bf16* __restrict__ vc, const int* __restrict__ block_tables, const int* __restrict__ seg,
                  const int* __restrict__ pos, const int* __restrict__ tiles, int nh, int nkv, int page,
                  int max_blocks, int q_stride, int out_stride, float scale_log2e, int window) {
     constexpr int D = D16 * 16;
     constexpr int KS = (D + 31) / 32;
-    constexpr int KROW = D + 8;    // padded rows: conflict-free 16-byte reads of 16 rows
-    constexpr int VROW = 32 + 8;
-    __shared__ __attribute__((aligned(16))) bf16 Ks[2][32][KROW];
-    __shared__ __attribute__((aligned(16))) bf16 Vs[2][D][VROW];
-    const int t0 = tiles[2 * blockIdx.x], ntok = tiles[2 * blockIdx.x + 1];
+    constexpr int KROW = D + 8;         // padded rows: conflict-free 16-byte reads of 16 rows
+    constexpr int VROW = ATT_TK + 8;
+    __shared__ __attribute__((aligned(16))) bf16 Ks[ATT_TK][KROW];
+    __shared__ __attribute__((aligned(16))) bf16 Vs[D][VROW];
+    __shared__ int bt_s[ATT_BT_LDS];
+    // the longest tiles (latest positions) are dispatched first
+    const int tile_id = gridDim.x - 1 - blockIdx.x;
+    const int t0 = tiles[2 * tile_id], ntok = tiles[2 * tile_id + 1];
     const int G = nh / nkv;
     const int HG = (G + 15) / 16;
     const int kvh = blockIdx.y / HG, hg = blockIdx.y % HG;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, qg = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, qg = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: what depends on it stays in SGPRs
     const int hcol = hg * 16 + r;
     const bool head_ok = hcol < G;
     const int head = kvh * G + (head_ok ? hcol : G - 1);
@@ -310,6 +321,13 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     const int lo_first = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
     const int* bt = block_tables + (size_t)seg[t0] * max_blocks;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+
+    // the pages of the keys this tile sees, into LDS (page lookups then cost no trip to memory)
+    const int blk_first = lo_first / page, blk_count = p_last / page - blk_first + 1;
+    const bool bt_in_lds = blk_count <= ATT_BT_LDS;
+    if (bt_in_lds)
+        for (int i = tid; i < blk_count; i += 256) bt_s[i] = bt[blk_first + i];
+    auto page_of = [&](int key) -> int { return bt_in_lds ? bt_s[key / page - blk_first] : bt[key / page]; };
 
     // this wave's tokens
     int tok[ATT_NT], pj[ATT_NT], loj[ATT_NT];
@@ -340,101 +358,152 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
         for (int db = 0; db < D16; ++db) acc[j][db] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // cooperative copy of one 32-key tile: K rows [key][d], V rows [d][key]
-    constexpr int KPIECES = 32 * (D / 8);   // 16-byte pieces
-    constexpr int VPIECES = D * 4;
+    // cooperative copy of one tile of ATT_TK keys: K rows [key][d], V rows [d][key], 16-byte pieces
+    constexpr int KPIECES = ATT_TK * (D / 8);
+    constexpr int VPIECES = D * (ATT_TK / 8);
     constexpr int KPER = (KPIECES + 255) / 256, VPER = (VPIECES + 255) / 256;
-    static_assert(KPER <= 2 && VPER <= 2, "a tile is at most two 16-byte pieces a thread");
+    static_assert(KPER <= 4 && VPER <= 4, "a tile is at most four 16-byte pieces a thread");
+    // PAGE64: the page size is a multiple of the tile's 64 keys, so a tile lies on one page: one page
+    // lookup a tile (the same for every thread) and no clamping - keys of the page beyond the tokens'
+    // reach are masked later.  Otherwise every piece finds its own page.
+    int koff[4], voff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int pk = tid + i * 256 < KPIECES ? tid + i * 256 : 0;
+        const int pv = tid + i * 256 < VPIECES ? tid + i * 256 : 0;
+        koff[i] = (pk / (D / 8)) * D + (pk % (D / 8)) * 8;
+        voff[i] = (pv / (ATT_TK / 8)) * page + (pv % (ATT_TK / 8)) * 8;
+    }
+    const bf16* ktile = kc;
+    const bf16* vtile = vc;
     auto fetch_k = [&](int kb, int i) -> uint4 {
+        if (PAGE64) return *reinterpret_cast<const uint4*>(ktile + koff[i]);
         const int pc = tid + i * 256;
         const int row = (pc < KPIECES ? pc : 0) / (D / 8), col = (pc < KPIECES ? pc : 0) % (D / 8);
         int key = kb + row;
         key = key < lo_first ? lo_first : (key > p_last ? p_last : key);   // a page that exists
-        const int pg = bt[key / page];
+        const int pg = page_of(key);
         return *reinterpret_cast<const uint4*>(kc + (((size_t)pg * nkv + kvh) * page + (key % page)) * D + col * 8);
     };
     auto fetch_v = [&](int kb, int i) -> uint4 {
+        if (PAGE64) return *reinterpret_cast<const uint4*>(vtile + voff[i]);
         const int pc = tid + i * 256;
-        const int drow = (pc < VPIECES ? pc : 0) >> 2, kgrp = (pc < VPIECES ? pc : 0) & 3;
+        const int drow = (pc < VPIECES ? pc : 0) / (ATT_TK / 8), kgrp = (pc < VPIECES ? pc : 0) % (ATT_TK / 8);
         int key0 = kb + kgrp * 8;
         if (key0 > p_last || key0 + 8 <= lo_first) key0 = lo_first & ~7;   // masked later; any valid group
-        const int pg = bt[key0 / page];
+        const int pg = page_of(key0);
         return *reinterpret_cast<const uint4*>(vc + (((size_t)pg * nkv + kvh) * D + drow) * page + (key0 % page));
     };
-    auto stash_k = [&](int buf, int i, uint4 v) {
+    auto stash_k = [&](int i, uint4 v) {
         const int pc = tid + i * 256;
-        if (pc < KPIECES) *reinterpret_cast<uint4*>(&Ks[buf][pc / (D / 8)][(pc % (D / 8)) * 8]) = v;
+        if (pc < KPIECES) *reinterpret_cast<uint4*>(&Ks[pc / (D / 8)][(pc % (D / 8)) * 8]) = v;
     };
-    auto stash_v = [&](int buf, int i, uint4 v) {
+    auto stash_v = [&](int i, uint4 v) {
         const int pc = tid + i * 256;
-        if (pc < VPIECES) *reinterpret_cast<uint4*>(&Vs[buf][pc >> 2][(pc & 3) * 8]) = v;
+        if (pc < VPIECES) *reinterpret_cast<uint4*>(&Vs[pc / (ATT_TK / 8)][(pc % (ATT_TK / 8)) * 8]) = v;
     };
-    uint4 k0 = zero4, k1 = zero4, v0 = zero4, v1 = zero4;
+    uint4 k0 = zero4, k1 = zero4, k2 = zero4, k3 = zero4, v0 = zero4, v1 = zero4, v2 = zero4, v3 = zero4;
 #define ATT_FETCH(kb_)                          \
+    if (PAGE64) {                               \
+        const int pg_ = page_of(kb_);           \
+        ktile = kc + (((size_t)pg_ * nkv + kvh) * page + ((kb_) % page)) * D; \
+        vtile = vc + ((size_t)pg_ * nkv + kvh) * D * page + ((kb_) % page);   \
+    }                                           \
     k0 = fetch_k(kb_, 0);                       \
     if (KPER > 1) k1 = fetch_k(kb_, 1);         \
+    if (KPER > 2) k2 = fetch_k(kb_, 2);         \
+    if (KPER > 3) k3 = fetch_k(kb_, 3);         \
     v0 = fetch_v(kb_, 0);                       \
-    if (VPER > 1) v1 = fetch_v(kb_, 1);
-#define ATT_STASH(buf_)                         \
-    stash_k(buf_, 0, k0);                       \
-    if (KPER > 1) stash_k(buf_, 1, k1);         \
-    stash_v(buf_, 0, v0);                       \
-    if (VPER > 1) stash_v(buf_, 1, v1);
+    if (VPER > 1) v1 = fetch_v(kb_, 1);         \
+    if (VPER > 2) v2 = fetch_v(kb_, 2);         \
+    if (VPER > 3) v3 = fetch_v(kb_, 3);
+#define ATT_STASH()                             \
+    stash_k(0, k0);                             \
+    if (KPER > 1) stash_k(1, k1);               \
+    if (KPER > 2) stash_k(2, k2);               \
+    if (KPER > 3) stash_k(3, k3);               \
+    stash_v(0, v0);                             \
+    if (VPER > 1) stash_v(1, v1);               \
+    if (VPER > 2) stash_v(2, v2);               \
+    if (VPER > 3) stash_v(3, v3);
 
-    const int kb0 = lo_first & ~31;
+    const int kb0 = lo_first & ~(ATT_TK - 1);
+    __syncthreads();   // bt_s is filled
     ATT_FETCH(kb0)
-    ATT_STASH(0)
-    __syncthreads();
-    int buf = 0;
-    for (int kb = kb0; kb <= p_last; kb += 32, buf ^= 1) {
-        const bool more = kb + 32 <= p_last;
-        if (more) { ATT_FETCH(kb + 32) }
-        // ---- this wave's tokens against the tile in Ks[buf], Vs[buf]
-        const bool any = kb <= pj[ATT_NT - 1] && kb + 32 > loj[0];   // wave-uniform
-        if (any) {
+    for (int kb = kb0; kb <= p_last; kb += ATT_TK) {
+        __syncthreads();   // the previous tile has been consumed
+        ATT_STASH()
+        __syncthreads();
+        if (kb + ATT_TK <= p_last) { ATT_FETCH(kb + ATT_TK) }   // in flight while this tile is multiplied
+#pragma unroll
+        for (int sub = 0; sub < ATT_TK / 32; ++sub) {
+            const int kbs = kb + sub * 32;
+            const bool any = kbs <= pj[ATT_NT - 1] && kbs + 32 > loj[0];   // wave-uniform
+            if (!any) continue;
+            // four independent accumulator chains (2 key tiles x 2 tokens), interleaved over d
             f32x4 s[ATT_NT][2];
+            uint4 kf[2][KS];
 #pragma unroll
             for (int tau = 0; tau < 2; ++tau) {
-                const int row = (r >> 2) * 8 + tau * 4 + (r & 3);
-                uint4 kf[KS];
+                const int row = sub * 32 + (r >> 2) * 8 + tau * 4 + (r & 3);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     const int dofs = ks * 32 + qg * 8;
-                    kf[ks] = dofs < D ? *reinterpret_cast<const uint4*>(&Ks[buf][row][dofs]) : zero4;
+                    kf[tau][ks] = (D % 32 == 0 || dofs < D)
+                                      ? *reinterpret_cast<const uint4*>(&Ks[row][D % 32 == 0 ? dofs : (dofs < D ? dofs : 0)])
+                                      : zero4;
                 }
 #pragma unroll
-                for (int j = 0; j < ATT_NT; ++j) {
-                    s[j][tau] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) s[j][tau] = mfma16(kf[ks], qf[j][ks], s[j][tau]);
-                }
+                for (int j = 0; j < ATT_NT; ++j) s[j][tau] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
-            uint4 pf[ATT_NT];
-            float corr[ATT_NT];
 #pragma unroll
-            for (int j = 0; j < ATT_NT; ++j) {
-                float sv[8];
-                float mx = NEG_BIG;
+            for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                 for (int tau = 0; tau < 2; ++tau)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int key = kb + qg * 8 + tau * 4 + e;
-                        const bool ok = key >= loj[j] && key <= pj[j];
-                        const float v = ok ? s[j][tau][e] * scale_log2e : NEG_BIG;
-                        sv[tau * 4 + e] = v;
-                        mx = fmaxf(mx, v);
+                    for (int j = 0; j < ATT_NT; ++j) s[j][tau] = mfma16(kf[tau][ks], qf[j][ks], s[j][tau]);
+            // Softmax on raw scores: the scale enters the exponent's multiply-add.  Sub-tiles that
+            // every token of the wave sees whole (all but those on the diagonal or a window's edge)
+            // skip the masks, and the accumulators are rescaled only when some row's maximum moved.
+            uint4 pf[ATT_NT];
+            float corr[ATT_NT];
+            const bool full = kbs + 31 <= pj[0] && kbs >= loj[ATT_NT - 1];   // wave-uniform
+            bool moved = false;
+#pragma unroll
+            for (int j = 0; j < ATT_NT; ++j) {
+                float sv[8];
+#pragma unroll
+                for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) sv[tau * 4 + e] = s[j][tau][e];
+                if (!full) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const int key = kbs + qg * 8 + i;
+                        sv[i] = (key >= loj[j] && key <= pj[j]) ? sv[i] : NEG_BIG;
                     }
+                }
+                float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
                 mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
                 mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
                 const float m_new = fmaxf(m[j], mx);
-                corr[j] = __builtin_amdgcn_exp2f(m[j] - m_new);
+                corr[j] = (m_new > m[j]) ? __builtin_amdgcn_exp2f((m[j] - m_new) * scale_log2e) : 1.0f;
+                moved = moved || (m_new > m[j]);
+                const float mc = m_new * scale_log2e;
                 float pe[8];
                 float rs = 0.f;
+                if (full) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    pe[i] = (sv[i] > 0.5f * NEG_BIG) ? __builtin_amdgcn_exp2f(sv[i] - m_new) : 0.f;
-                    rs += pe[i];
+                    for (int i = 0; i < 8; ++i) {
+                        pe[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, -mc));
+                        rs += pe[i];
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        pe[i] = (sv[i] > 0.5f * NEG_BIG) ? __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, -mc)) : 0.f;
+                        rs += pe[i];
+                    }
                 }
                 rs += __shfl_xor(rs, 16, 64);
                 rs += __shfl_xor(rs, 32, 64);
@@ -445,22 +514,24 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
                 pf[j].z = pack_bf16x2(pe[4], pe[5]);
                 pf[j].w = pack_bf16x2(pe[6], pe[7]);
             }
-            const int key0 = kb + qg * 8;
+            if (__builtin_amdgcn_ballot_w64(moved) != 0ull) {
+#pragma unroll
+                for (int j = 0; j < ATT_NT; ++j)
+#pragma unroll
+                    for (int db = 0; db < D16; ++db)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[j][db][e] *= corr[j];
+            }
+            const int key0 = kbs + qg * 8;
             const bool vok = key0 <= p_last && key0 + 8 > lo_first;   // else the tile holds another group's values
 #pragma unroll
             for (int db = 0; db < D16; ++db) {
-                const uint4 v = *reinterpret_cast<const uint4*>(&Vs[buf][db * 16 + r][qg * 8]);
-                const uint4 vf = vok ? v : zero4;
+                const uint4 v = *reinterpret_cast<const uint4*>(&Vs[db * 16 + r][sub * 32 + qg * 8]);
+                const uint4 vf = (PAGE64 || vok) ? v : zero4;   // PAGE64: the tile's own page, finite, times p = 0
 #pragma unroll
-                for (int j = 0; j < ATT_NT; ++j) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[j][db][e] *= corr[j];
-                    acc[j][db] = mfma16(vf, pf[j], acc[j][db]);
-                }
+                for (int j = 0; j < ATT_NT; ++j) acc[j][db] = mfma16(vf, pf[j], acc[j][db]);
             }
         }
-        if (more) { ATT_STASH(buf ^ 1) }
-        __syncthreads();
     }
     if (!head_ok) return;
 #pragma unroll
@@ -496,18 +567,19 @@ extern "C" int ilm_attn_tile(void* out, const void* q, const void* kc, const voi
     ILM_REQUIRE(nkv * HG <= 65535, "attn_tile: grid too large");
     dim3 grid(n_tiles, nkv * HG);
     const float sl2 = scale * 1.4426950408889634f;
-#define AT_CASE(D16)                                                                                            \
-    case D16:                                                                                                   \
-        attn_tile_kernel<D16><<<grid, 256, 0, stream>>>((bf16*)out, (const bf16*)q, (const bf16*)kc, (const bf16*)vc, \
-                                                        (const int*)block_tables, (const int*)seg, (const int*)pos, \
-                                                        (const int*)tiles, nh, nkv, page, max_blocks, q_stride, \
-                                                        out_stride, sl2, window);                               \
+#define AT_ARGS (bf16*)out, (const bf16*)q, (const bf16*)kc, (const bf16*)vc, (const int*)block_tables, (const int*)seg, \
+                (const int*)pos, (const int*)tiles, nh, nkv, page, max_blocks, q_stride, out_stride, sl2, window
+#define AT_CASE(D16)                                                                   \
+    case D16:                                                                          \
+        if (page % ATT_TK == 0) attn_tile_kernel<D16, true><<<grid, 256, 0, stream>>>(AT_ARGS);  \
+        else attn_tile_kernel<D16, false><<<grid, 256, 0, stream>>>(AT_ARGS);          \
         break
     switch (d / 16) {
         AT_CASE(1); AT_CASE(2); AT_CASE(3); AT_CASE(4); AT_CASE(5); AT_CASE(6); AT_CASE(7); AT_CASE(8);
         default: ILM_REQUIRE(false, "attn_tile: head size %d", d);
     }
 #undef AT_CASE
+#undef AT_ARGS
     ILM_LAUNCH_CHECK("attn_tile");
     return 0;
 }

@@ -48,8 +48,9 @@ __device__ __forceinline__ float from_f32<float>(float v) {
 }
 template <>
 __device__ __forceinline__ bf16 from_f32<bf16>(float v) {
+    // the hardware's conversion (round to nearest even), one instruction on gfx950
     bf16 r;
-    r.bits = f32_to_bf16_bits(v);
+    r.bits = __builtin_bit_cast(uint16_t, (__bf16)v);
     return r;
 }
 
