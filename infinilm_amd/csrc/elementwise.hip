@@ -45,16 +45,18 @@ extern "C" int ilm_embed(void* r, const void* ids, const void* table, int T_, in
 // One block per row.  The sum of squares is reduced in an order that depends on H only, so a
 // row's result does not depend on what else is in the batch.
 // ------------------------------------------------------------------------------------------
-template <typename T, typename WT>
+template <typename T, typename WT, typename HT>
 __global__ void __launch_bounds__(256)
-add_rmsnorm_kernel(T* __restrict__ x, float* __restrict__ r, const T* __restrict__ h,
-                   const WT* __restrict__ w, int H, float alpha, float eps) {
+add_rmsnorm_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __restrict__ h,
+                   const WT* __restrict__ w, int H, float alpha, float eps, int parts, size_t pstride) {
     __shared__ float red[4];
     const size_t base = (size_t)blockIdx.x * H;
     float ss = 0.f;
     if (h != nullptr) {
         for (int j = threadIdx.x; j < H; j += 256) {
-            float v = r[base + j] + alpha * to_f32(h[base + j]);
+            float hs = 0.f;
+            for (int p = 0; p < parts; ++p) hs += to_f32(h[p * pstride + base + j]);
+            float v = r[base + j] + alpha * hs;
             r[base + j] = v;
             ss += v * v;
         }
@@ -73,10 +75,10 @@ add_rmsnorm_kernel(T* __restrict__ x, float* __restrict__ r, const T* __restrict
 // Fast form for H = 8 * 256 * NITER' (NITER' <= NITER): each thread keeps its 8 * NITER values in
 // registers between the sum of squares and the scaling, and moves 16 or 32 bytes per access.
 // The order of the sum depends on H only.
-template <typename T, typename WT, int NITER>
+template <typename T, typename WT, typename HT, int NITER>
 __global__ void __launch_bounds__(256)
-add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const T* __restrict__ h,
-                       const WT* __restrict__ w, int H, float alpha, float eps) {
+add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __restrict__ h,
+                       const WT* __restrict__ w, int H, float alpha, float eps, int parts, size_t pstride) {
     __shared__ float red[4];
     const size_t base = (size_t)blockIdx.x * H;
     float v[NITER][8];
@@ -90,15 +92,21 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const T* __rest
             v[it][0] = r0.x; v[it][1] = r0.y; v[it][2] = r0.z; v[it][3] = r0.w;
             v[it][4] = r1.x; v[it][5] = r1.y; v[it][6] = r1.z; v[it][7] = r1.w;
             if (h != nullptr) {
-                T hv[8];
-                if (sizeof(T) == 2) {
-                    *reinterpret_cast<uint4*>(hv) = *reinterpret_cast<const uint4*>(h + base + j);
-                } else {
-                    *reinterpret_cast<float4*>(hv) = *reinterpret_cast<const float4*>(h + base + j);
-                    *reinterpret_cast<float4*>(hv + 4) = *reinterpret_cast<const float4*>(h + base + j + 4);
+                float hs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                for (int p = 0; p < parts; ++p) {   // parts of a K-split product, summed in order
+                    HT hv[8];
+                    const HT* hp = h + p * pstride + base + j;
+                    if (sizeof(HT) == 2) {
+                        *reinterpret_cast<uint4*>(hv) = *reinterpret_cast<const uint4*>(hp);
+                    } else {
+                        *reinterpret_cast<float4*>(hv) = *reinterpret_cast<const float4*>(hp);
+                        *reinterpret_cast<float4*>(hv + 4) = *reinterpret_cast<const float4*>(hp + 4);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) hs[e] += to_f32(hv[e]);
                 }
 #pragma unroll
-                for (int e = 0; e < 8; ++e) v[it][e] += alpha * to_f32(hv[e]);
+                for (int e = 0; e < 8; ++e) v[it][e] += alpha * hs[e];
                 *reinterpret_cast<float4*>(r + base + j) = make_float4(v[it][0], v[it][1], v[it][2], v[it][3]);
                 *reinterpret_cast<float4*>(r + base + j + 4) = make_float4(v[it][4], v[it][5], v[it][6], v[it][7]);
             }
@@ -125,29 +133,42 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const T* __rest
     }
 }
 
+// h: the pending branch [parts][rows][H] in the activations' dtype (h_dtype == dtype) or in float
+// (h_dtype == ILM_DTYPE_F32, e.g. the parts of a K-split product); null: nothing to add.
 extern "C" int ilm_add_rmsnorm(void* x, void* r, const void* h, const void* w, int rows, int H,
-                               float alpha, float eps, int dtype, int w_dtype,
-                               hipStream_t stream) {
+                               float alpha, float eps, int dtype, int w_dtype, int h_dtype, int parts,
+                               long pstride, hipStream_t stream) {
     ILM_REQUIRE(rows > 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", rows, H);
+    ILM_REQUIRE(h == nullptr || (parts >= 1 && (h_dtype == dtype || h_dtype == ILM_DTYPE_F32)),
+                "add_rmsnorm: the branch must have the activations' dtype or be float, in >= 1 parts");
     // H a multiple of 8 up to 8192 with 16-byte aligned rows takes the vector kernel
     const bool vec = H % 8 == 0 && H <= 8192 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)r & 15) == 0 &&
-                     ((uintptr_t)h & 15) == 0;
+                     ((uintptr_t)h & 15) == 0 && pstride % 8 == 0;
     const int niter = (H + 2047) / 2048;
-#define NORM_CASE(T, WT)                                                                                        \
-    if (vec && niter <= 1)                                                                                      \
-        add_rmsnorm_vec_kernel<T, WT, 1><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const T*)h, (const WT*)w, H, alpha, eps); \
-    else if (vec && niter <= 2)                                                                                 \
-        add_rmsnorm_vec_kernel<T, WT, 2><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const T*)h, (const WT*)w, H, alpha, eps); \
-    else if (vec)                                                                                               \
-        add_rmsnorm_vec_kernel<T, WT, 4><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const T*)h, (const WT*)w, H, alpha, eps); \
-    else                                                                                                        \
-        add_rmsnorm_kernel<T, WT><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const T*)h, (const WT*)w, H, alpha, eps)
+    const bool hf = h != nullptr && h_dtype == ILM_DTYPE_F32;
+#define NORM_LAUNCH(T, WT, HT)                                                                                   \
+    do {                                                                                                         \
+        if (vec && niter <= 1)                                                                                   \
+            add_rmsnorm_vec_kernel<T, WT, HT, 1><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride); \
+        else if (vec && niter <= 2)                                                                              \
+            add_rmsnorm_vec_kernel<T, WT, HT, 2><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride); \
+        else if (vec)                                                                                            \
+            add_rmsnorm_vec_kernel<T, WT, HT, 4><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride); \
+        else                                                                                                     \
+            add_rmsnorm_kernel<T, WT, HT><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride); \
+    } while (0)
+#define NORM_CASE(T, WT)                     \
+    do {                                     \
+        if (hf) NORM_LAUNCH(T, WT, float);   \
+        else NORM_LAUNCH(T, WT, T);          \
+    } while (0)
     if (dtype == ILM_DTYPE_F32 && w_dtype == ILM_DTYPE_F32) NORM_CASE(float, float);
     else if (dtype == ILM_DTYPE_BF16 && w_dtype == ILM_DTYPE_BF16) NORM_CASE(bf16, bf16);
     else if (dtype == ILM_DTYPE_BF16 && w_dtype == ILM_DTYPE_F32) NORM_CASE(bf16, float);
     else if (dtype == ILM_DTYPE_F32 && w_dtype == ILM_DTYPE_BF16) NORM_CASE(float, bf16);
     else ILM_REQUIRE(false, "add_rmsnorm: unknown dtypes %d %d", dtype, w_dtype);
 #undef NORM_CASE
+#undef NORM_LAUNCH
     ILM_LAUNCH_CHECK("add_rmsnorm");
     return 0;
 }

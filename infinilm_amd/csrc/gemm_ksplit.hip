@@ -1,0 +1,135 @@
+// The decode-side projection (at most 16 rows of X, bfloat16) for long K: blockIdx.y takes a
+// contiguous K range of GF_KSPAN and writes a float partial result C[y][M][N]; the consumer (the next
+// add+RMSNorm) sums the parts in order.  Within a range the kernel is the resident few-rows
+// product: W streamed once on v_mfma_f32_16x16x32_bf16, the X fragments in registers, the next W
+// row tile prefetched while the previous one is reduced.  This gives the long-K product
+// (down_proj) the shape of the short-K ones instead of 64 k-steps a wave.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+#define GF_KSPAN 4096   // K a workgroup covers: waves x k-steps x 32
+
+__device__ __forceinline__ f32x4 gf_mfma(uint4 a, uint4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+// 16 waves x 8 k-steps keep a wave under 128 registers (4 waves a SIMD, one workgroup a CU).
+template <int GF_WAVES, int GF_KSTEPS, typename TC>
+__global__ void __launch_bounds__(GF_WAVES * 64)
+gemm_ksplit_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
+                   const bf16* __restrict__ bias, int M, int N, int K, int lda, int ldw, int ldc, float alpha,
+                   int ntiles, size_t c_part_stride) {
+    __shared__ float part[2][GF_WAVES][64][4];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = lane & 15, q = lane >> 4;
+    const int kslice = blockIdx.y;
+    static_assert(GF_WAVES * GF_KSTEPS * 32 == GF_KSPAN, "a workgroup covers GF_KSPAN of K");
+    const int k_lo = kslice * GF_KSPAN;           // this workgroup's K range starts here
+    const int k_hi = (k_lo + GF_KSPAN < K) ? k_lo + GF_KSPAN : K;
+    const int s0 = wave * GF_KSTEPS;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    const int k8_first = k_lo >> 3, k8_last = (k_hi >> 3) - 1;
+    int k8c[GF_KSTEPS];
+    bool kok[GF_KSTEPS];
+#pragma unroll
+    for (int u = 0; u < GF_KSTEPS; ++u) {
+        const int k8 = k8_first + (s0 + u) * 4 + q;
+        kok[u] = k8 <= k8_last;
+        k8c[u] = kok[u] ? k8 : k8_last;
+    }
+    // the first W tile is on its way before anything else
+    uint4 a[GF_KSTEPS];
+    int tile = blockIdx.x;
+    if (tile < ntiles) {
+        const int row = (tile * 16 + r < N) ? tile * 16 + r : N - 1;
+        const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)row * ldw);
+#pragma unroll
+        for (int u = 0; u < GF_KSTEPS; ++u) a[u] = wp[k8c[u]];
+    }
+    uint4 xf[GF_KSTEPS];
+    const bool row_ok = r < M;
+    {
+        const uint4* xp = reinterpret_cast<const uint4*>(X + (size_t)(row_ok ? r : 0) * lda);
+#pragma unroll
+        for (int u = 0; u < GF_KSTEPS; ++u) {
+            const uint4 v = xp[k8c[u]];
+            xf[u] = (kok[u] && row_ok) ? v : zero;   // zero fragments make the clamped W loads harmless
+        }
+    }
+    TC* Cp = C + (size_t)kslice * c_part_stride;
+    int buf = 0;
+    for (; tile < ntiles; tile += gridDim.x) {
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < GF_KSTEPS; ++u) acc = gf_mfma(a[u], xf[u], acc);
+        const int next = tile + gridDim.x;
+        __builtin_amdgcn_sched_barrier(0);
+        if (next < ntiles) {   // the next tile's rows are on their way while this one is reduced
+            const int row = (next * 16 + r < N) ? next * 16 + r : N - 1;
+            const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)row * ldw);
+#pragma unroll
+            for (int u = 0; u < GF_KSTEPS; ++u) a[u] = wp[k8c[u]];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        *reinterpret_cast<f32x4*>(&part[buf][wave][lane][0]) = acc;
+        __syncthreads();
+        if (threadIdx.x < 256) {
+            const int e = threadIdx.x & 3, l = threadIdx.x >> 2;
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < GF_WAVES; ++w) v += part[buf][w][l][e];
+            const int n = tile * 16 + (l >> 4) * 4 + e;
+            const int m = l & 15;
+            if (n < N && m < M) {
+                if (bias != nullptr && kslice == 0) v += to_f32(bias[n]);
+                Cp[(size_t)m * ldc + n] = from_f32<TC>(alpha * v);
+            }
+        }
+        buf ^= 1;  // the other buffer is free: its readers passed the barrier above one tile ago
+    }
+}
+
+static int gf_num_cus() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
+// Largest K a call takes, given how many parts the caller lets the result be split into.
+extern "C" int ilm_gemm_ksplit_max_k(int parts) { return GF_KSPAN * parts; }
+
+// kb > 1: C must be float, [kb][M][ldc] with c_part_stride elements between the parts.
+extern "C" int ilm_gemm_ksplit(void* C, int out_dtype, int ldc, long c_part_stride, int kb, const void* W, int ldw,
+                               const void* bias, float alpha, int M, int N, int K, const void* X, int lda,
+                               hipStream_t stream) {
+    ILM_REQUIRE(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_ksplit: needs 1 <= M <= 16, got M=%d N=%d K=%d", M, N, K);
+    ILM_REQUIRE(K % 8 == 0 && ldw % 8 == 0 && ldw >= K && ldc >= N, "gemm_ksplit: K=%d ldw=%d ldc=%d", K, ldw, ldc);
+    ILM_REQUIRE(kb >= 1 && K <= ilm_gemm_ksplit_max_k(kb), "gemm_ksplit: K=%d does not fit %d parts of %d", K, kb,
+                GF_KSPAN);
+    ILM_REQUIRE(kb == 1 || out_dtype == ILM_DTYPE_F32, "gemm_ksplit: partial results are float");
+    ILM_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && lda % 8 == 0 && lda >= K,
+                "gemm_ksplit: X and W rows must be 16-byte aligned");
+    const int ntiles = (N + 15) / 16;
+    int gx = gf_num_cus() / kb;
+    if (gx < 1) gx = 1;
+    if (gx > ntiles) gx = ntiles;
+    dim3 grid(gx, kb);
+    if (out_dtype == ILM_DTYPE_BF16)
+        gemm_ksplit_kernel<16, 8, bf16><<<grid, 16 * 64, 0, stream>>>((bf16*)C, (const bf16*)X, (const bf16*)W,
+                                                                      (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha,
+                                                                      ntiles, (size_t)c_part_stride);
+    else if (out_dtype == ILM_DTYPE_F32)
+        gemm_ksplit_kernel<16, 8, float><<<grid, 16 * 64, 0, stream>>>((float*)C, (const bf16*)X, (const bf16*)W,
+                                                                       (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha,
+                                                                       ntiles, (size_t)c_part_stride);
+    else
+        ILM_REQUIRE(false, "gemm_ksplit: unknown output dtype %d", out_dtype);
+    ILM_LAUNCH_CHECK("gemm_ksplit");
+    return 0;
+}

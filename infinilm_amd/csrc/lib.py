@@ -8,7 +8,7 @@ time, the kernels raise.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_float, c_int, c_void_p
+from ctypes import c_float, c_int, c_long, c_void_p
 from typing import Optional
 
 _lib: Optional[ctypes.CDLL] = None
@@ -16,10 +16,12 @@ _lib: Optional[ctypes.CDLL] = None
 _P = c_void_p
 _I = c_int
 _F = c_float
+_L = c_long
 
 _SIGNATURES = {
     "ilm_embed": [_P, _P, _P, _I, _I, _I, _F, _I, _P],
-    "ilm_add_rmsnorm": [_P, _P, _P, _P, _I, _I, _F, _F, _I, _I, _P],
+    "ilm_add_rmsnorm": [_P, _P, _P, _P, _I, _I, _F, _F, _I, _I, _I, _I, _L, _P],
+    "ilm_gemm_ksplit": [_P, _I, _I, _L, _I, _P, _I, _P, _F, _I, _I, _I, _P, _I, _P],
     "ilm_rope_kvwrite": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "ilm_swiglu": [_P, _P, _I, _I, _I, _I, _P],
     "ilm_gather_rows": [_P, _P, _P, _I, _I, _I, _P],

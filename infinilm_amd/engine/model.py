@@ -91,7 +91,12 @@ class CausalLM:
         if not batch.wants_all_rows:
             last = ResidualStream(kernels.gather_rows(stream.residual, batch.want_rows))
             if stream.pending is not None:
-                last.push(kernels.gather_rows(stream.pending, batch.want_rows), stream.pending_scale)
+                pend = stream.pending
+                if pend.dim() == 3:   # parts of a K-split product: the rows of every part
+                    pend = torch.stack([kernels.gather_rows(p, batch.want_rows) for p in pend])
+                else:
+                    pend = kernels.gather_rows(pend, batch.want_rows)
+                last.push(pend, stream.pending_scale)
             stream = last
         x = self.final_norm.forward(stream)
         return kernels.gemm(x, self.head, None, self.spec.head.scale, torch.float32)

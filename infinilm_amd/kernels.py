@@ -22,6 +22,7 @@ ATT_CHUNK = 256  # keys per chunk of the matrix-core attention kernel (ilm_attn_
 # INFINILM_AMD_BASIC=1 runs the plain kernels everywhere (for telling a kernel's fault from the engine's)
 FORCE_BASIC = os.environ.get("INFINILM_AMD_BASIC", "0") == "1"
 SKINNY_VARIANT = int(os.environ.get("INFINILM_AMD_SKINNY_VARIANT", "0"))  # 0: the kernel chooses
+USE_KSPLIT = os.environ.get("INFINILM_AMD_KSPLIT", "1") == "1"
 USE_LIBRARY_GEMM = os.environ.get("INFINILM_AMD_LIBRARY_GEMM", "1") == "1"
 
 
@@ -91,18 +92,27 @@ def embed(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
 
 def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: torch.Tensor,
                 alpha: float, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
-    """residual += alpha * branch (in place, float32), then its RMS norm times weight, as out_dtype."""
+    """residual += alpha * branch (in place, float32), then its RMS norm times weight, as out_dtype.
+
+    `branch` is [rows, H] in out_dtype or float32, or [parts, rows, H] (the float32 parts of a K-split
+    product, summed in order)."""
     _dev(residual, branch, weight)
     rows, H = residual.shape
     if residual.dtype != F32 or not residual.is_contiguous():
         raise KernelError("the residual stream is a contiguous float32 tensor")
-    if branch is not None and (branch.shape != residual.shape or branch.dtype != out_dtype or not branch.is_contiguous()):
-        raise KernelError(f"branch {tuple(branch.shape)} {branch.dtype} does not match residual {tuple(residual.shape)} / {out_dtype}")
+    parts, pstride, h_dt = 1, 0, _DT[out_dtype]
+    if branch is not None:
+        if branch.dim() == 3:
+            parts, pstride = branch.shape[0], branch.stride(0)
+        if tuple(branch.shape[-2:]) != (rows, H) or branch.dtype not in (out_dtype, F32) or not branch.is_contiguous():
+            raise KernelError(f"branch {tuple(branch.shape)} {branch.dtype} does not match residual "
+                              f"{tuple(residual.shape)} / {out_dtype}")
+        h_dt = _dt(branch)
     if weight.shape != (H,) or not weight.is_contiguous():
         raise KernelError(f"norm weight has shape {tuple(weight.shape)}, expected ({H},)")
     out = torch.empty((rows, H), dtype=out_dtype, device=residual.device)
     _run("ilm_add_rmsnorm", out.data_ptr(), residual.data_ptr(), _ptr(branch), weight.data_ptr(), rows, H,
-         float(alpha), float(eps), _DT[out_dtype], _dt(weight), _stream())
+         float(alpha), float(eps), _DT[out_dtype], _dt(weight), h_dt, parts, pstride, _stream())
     return out
 
 
@@ -149,9 +159,16 @@ def gather_rows(x: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
     return out
 
 
+KSPLIT_SPAN = 4096  # K range of one part of the K-split few-rows product (ilm_gemm_ksplit_max_k(1))
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, alpha: float = 1.0,
-         out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """alpha * (a w^T + bias); a [M, K] with dense rows, w [N, K]; float accumulation."""
+         out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
+         allow_parts: bool = False) -> torch.Tensor:
+    """alpha * (a w^T + bias); a [M, K] with dense rows, w [N, K]; float accumulation.
+
+    `allow_parts`: the caller takes a float32 result in parts [P, M, N] that still have to be summed
+    (add_rmsnorm does); chosen for few rows and long K, where splitting K over workgroups pays."""
     _dev(a, w, bias, out)
     if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
         raise KernelError(f"gemm shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
@@ -162,25 +179,32 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     out_dtype = out_dtype or a.dtype
     if bias is not None and (bias.shape != (N,) or bias.dtype != w.dtype or not bias.is_contiguous()):
         raise KernelError(f"bias shape {tuple(bias.shape)} does not fit {N} outputs")
+    if out is not None and (out.shape != (M, N) or out.dtype != out_dtype or out.stride(1) != 1):
+        raise KernelError("gemm output does not fit")
+    fast = a.dtype == BF16 and not FORCE_BASIC
+    aligned = K % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 \
+        and w.data_ptr() % 16 == 0
+    plain = bias is None and alpha == 1.0
+    if fast and aligned and plain and allow_parts and out is None and M <= 16 and K > 2 * KSPLIT_SPAN and USE_KSPLIT:
+        kb = -(-K // KSPLIT_SPAN)
+        parts = torch.empty((kb, M, N), dtype=F32, device=a.device)
+        _run("ilm_gemm_ksplit", parts.data_ptr(), _DT[F32], N, M * N, kb, w.data_ptr(), w.stride(0), None, 1.0,
+             M, N, K, a.data_ptr(), a.stride(0), _stream())
+        return parts
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    elif out.shape != (M, N) or out.dtype != out_dtype or out.stride(1) != 1:
-        raise KernelError("gemm output does not fit")
-    if a.dtype == BF16 and not FORCE_BASIC:
-        aligned = K % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 \
-            and w.data_ptr() % 16 == 0
-        library_ok = bias is None and alpha == 1.0 and out_dtype == BF16 and USE_LIBRARY_GEMM
-        # measured at the 8B shapes: the few-rows kernel beats the vendor library up to 16 rows and
-        # loses to it above (its X fragments are re-read from L2 for every 16 rows of W)
-        if M <= 64 and aligned and not (M > 16 and library_ok):
-            _run("ilm_gemm_skinny", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
-                 w.stride(0), out.stride(0), float(alpha), _DT[out_dtype], SKINNY_VARIANT, _stream())
-            return out
-        if M > 16 and library_ok:
-            # large products go to the vendor library, as the reference's linear layers do
-            # (csrc/layers/quantization/none_quantization.cpp:26-46 calls its library's linear)
-            torch.matmul(a, w.t(), out=out)
-            return out
+    library_ok = fast and plain and out_dtype == BF16 and USE_LIBRARY_GEMM
+    # measured at the 8B shapes: the few-rows kernel beats the vendor library up to 16 rows and loses
+    # to it above (its X fragments are re-read from L2 for every 16 rows of W)
+    if fast and aligned and M <= 64 and not (M > 16 and library_ok):
+        _run("ilm_gemm_skinny", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
+             w.stride(0), out.stride(0), float(alpha), _DT[out_dtype], SKINNY_VARIANT, _stream())
+        return out
+    if M > 16 and library_ok:
+        # large products go to the vendor library, as the reference's linear layers do
+        # (csrc/layers/quantization/none_quantization.cpp:26-46 calls its library's linear)
+        torch.matmul(a, w.t(), out=out)
+        return out
     _run("ilm_gemm_basic", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0), w.stride(0),
          out.stride(0), float(alpha), _dt(a), _DT[out_dtype], _stream())
     return out

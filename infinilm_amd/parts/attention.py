@@ -55,4 +55,4 @@ class GQAttention(Mixer):
         o = kernels.paged_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,
                                     batch.positions, self.nh, self.nkv, self.d, self.scale, self.window,
                                     batch.max_total_len, batch.att_tiles, batch.att_single_rows)
-        return self.o_proj.forward(o)
+        return self.o_proj.forward(o, allow_parts=True)

@@ -51,7 +51,8 @@ class Part:
 
 class ResidualStream:
     """The residual stream in float32 and the branch output that is still to be added to it.
-    The sum `residual += scale * pending` happens inside the next norm's kernel."""
+    The sum `residual += scale * pending` happens inside the next norm's kernel.  `pending` is
+    [T, hidden] or, from a product that was split over K, float32 parts [P, T, hidden]."""
 
     def __init__(self, residual: torch.Tensor):
         self.residual = residual

@@ -37,8 +37,11 @@ class FusedLinear:
             row += size
         return out
 
-    def forward(self, x: torch.Tensor, alpha: float = 1.0, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-        return kernels.gemm(x, self.weight, self.bias, alpha, out_dtype)
+    def forward(self, x: torch.Tensor, alpha: float = 1.0, out_dtype: Optional[torch.dtype] = None,
+                allow_parts: bool = False) -> torch.Tensor:
+        """`allow_parts`: the result may come as float32 parts [P, T, out] still to be summed; only for a
+        result that goes straight into `ResidualStream.push` (the next norm's kernel sums them)."""
+        return kernels.gemm(x, self.weight, self.bias, alpha, out_dtype, allow_parts=allow_parts)
 
 
 class Linear(FusedLinear):

@@ -28,4 +28,4 @@ class SwiGLU(FeedForward):
         return out
 
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
-        return self.down.forward(kernels.swiglu(self.gate_up.forward(x)))
+        return self.down.forward(kernels.swiglu(self.gate_up.forward(x)), allow_parts=True)

@@ -144,6 +144,26 @@ def test_gemm_bfloat16(K, M, N, K_, out_dtype):
         _close(out, P.plain_linear(a.to(F64), w.to(F64), b.to(F64), 0.5), 1e-5 if out_dtype == torch.float32 else 6e-3)
 
 
+@pytest.mark.parametrize("M,N,K_", [(8, 4096, 16384), (1, 50, 8200), (16, 331, 12296)])
+def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
+    """Few rows and long K: the product comes as float32 parts; add_rmsnorm sums them in order."""
+    a, w = _rand((M, K_), 14, torch.bfloat16), _rand((N, K_), 15, torch.bfloat16, 0.05)
+    parts = K.gemm(a.to(DEV), w.to(DEV), allow_parts=True)
+    assert parts.dim() == 3 and parts.dtype == torch.float32 and parts.shape[0] == -(-K_ // 4096)
+    want = P.plain_linear(a.to(F64), w.to(F64))
+    _close(parts.sum(0), want, 1e-5)
+    whole = K.gemm(a.to(DEV), w.to(DEV))
+    assert whole.dim() == 2 and whole.dtype == torch.bfloat16
+    _close(whole, want, 6e-3)
+    r = _rand((M, N), 16, scale=2.0)
+    nw = _rand((N,), 17, torch.bfloat16) + 1
+    rd = r.to(DEV).clone()
+    x = K.add_rmsnorm(rd, parts, nw.to(DEV), 0.3, 1e-6, torch.bfloat16)
+    want_r = r.to(F64) + 0.3 * want
+    _close(rd, want_r, 1e-5)
+    _close(x, P.plain_rmsnorm(want_r, nw.to(F64), 1e-6), 1e-2)
+
+
 def _paged(k, v, page, n_pages, seed, dtype):
     """Scatters contiguous per-request keys/values [n, nkv, d] into a paged cache with a shuffled
     block table; unused slots hold large finite garbage so that a read beyond a length shows."""
