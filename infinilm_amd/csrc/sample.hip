@@ -28,7 +28,31 @@ __device__ __forceinline__ void better(float& bv, int& bi, float v, int i) {
 __device__ int block_argmax(const float* __restrict__ row, int V, float* sv, int* si, float* out_max) {
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += SB) better(bv, bi, row[i], i);
+    if ((V & 3) == 0 && ((uintptr_t)row & 15) == 0) {
+        // 16-byte loads, four of them in flight a thread: the scan is bound by memory latency
+        const float4* row4 = reinterpret_cast<const float4*>(row);
+        const int V4 = V >> 2;
+        for (int i = threadIdx.x; i < V4; i += 4 * SB) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = i + u * SB;
+                v[u] = row4[j < V4 ? j : V4 - 1];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = i + u * SB;
+                if (j < V4) {
+                    better(bv, bi, v[u].x, 4 * j);
+                    better(bv, bi, v[u].y, 4 * j + 1);
+                    better(bv, bi, v[u].z, 4 * j + 2);
+                    better(bv, bi, v[u].w, 4 * j + 3);
+                }
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < V; i += SB) better(bv, bi, row[i], i);
+    }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         float ov = __shfl_xor(bv, o, 64);

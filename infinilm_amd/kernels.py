@@ -167,8 +167,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
          allow_parts: bool = False) -> torch.Tensor:
     """alpha * (a w^T + bias); a [M, K] with dense rows, w [N, K]; float accumulation.
 
-    `allow_parts`: the caller takes a float32 result in parts [P, M, N] that still have to be summed
-    (add_rmsnorm does); chosen for few rows and long K, where splitting K over workgroups pays."""
+    `allow_parts`: the result goes straight into the residual sum (add_rmsnorm), so it may come in
+    float32 instead of the activations' dtype, and in parts [P, M, N] that still have to be summed;
+    parts are chosen for few rows and long K, where splitting K over workgroups pays."""
     _dev(a, w, bias, out)
     if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
         raise KernelError(f"gemm shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not fit")
@@ -191,6 +192,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
         _run("ilm_gemm_ksplit", parts.data_ptr(), _DT[F32], N, M * N, kb, w.data_ptr(), w.stride(0), None, 1.0,
              M, N, K, a.data_ptr(), a.stride(0), _stream())
         return parts
+    if fast and aligned and allow_parts and out is None and M <= 16:
+        out_dtype = F32   # a branch on its way into the float32 residual sum need not be rounded first
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     library_ok = fast and plain and out_dtype == BF16 and USE_LIBRARY_GEMM

@@ -249,3 +249,17 @@ def test_trace_run_program(models, tmp_path):
     assert rel_err(read(2), lb[[29]]) < TOL["float32"]
     assert rel_err(read(3), la[42:]) < TOL["float32"]
     assert rel_err(read(4), lb[[29]]) < TOL["float32"]
+
+
+def test_command_line(models):
+    """examples/test_infer.py with the reference's option names, token ids in place of a tokenizer."""
+    cfg, d, W = models[("A", "float32")]
+    prompt = random_tokens(cfg, 9, 5)
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "examples", "test_infer.py"), "--model", d, "--dtype", "float32",
+                           "--batch-size", "2", "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "7",
+                           "--top-k", "1", "--num-blocks", "16", "--block-size", "16", "--enable-paged-attn"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    want = str(P.plain_greedy(cfg, W, prompt, 7))
+    assert proc.stdout.count(want) == 2, proc.stdout[-1500:]
+    assert "total_time:" in proc.stdout

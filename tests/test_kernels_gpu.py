@@ -154,6 +154,8 @@ def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
     _close(parts.sum(0), want, 1e-5)
     whole = K.gemm(a.to(DEV), w.to(DEV))
     assert whole.dim() == 2 and whole.dtype == torch.bfloat16
+    short = K.gemm(a[:, :256].contiguous().to(DEV), w[:, :256].contiguous().to(DEV), allow_parts=True)
+    assert short.dim() == 2 and short.dtype == torch.float32   # short K: one part, not rounded to bfloat16
     _close(whole, want, 6e-3)
     r = _rand((M, N), 16, scale=2.0)
     nw = _rand((N,), 17, torch.bfloat16) + 1
