@@ -222,6 +222,89 @@ rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ pos, const floa
         for (int i = rd + threadIdx.x; i < d; i += 64) dst[i] = p[i];
 }
 
+// Vector form: one block a token, every thread 8 consecutive dims of a pair (16-byte accesses).
+// Needs rd a multiple of 16 (half the rotary dims in steps of 8) and d a multiple of 8.
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float* v) {
+    T t[8];
+    if (sizeof(T) == 2) {
+        *reinterpret_cast<uint4*>(t) = *reinterpret_cast<const uint4*>(p);
+    } else {
+        *reinterpret_cast<float4*>(t) = *reinterpret_cast<const float4*>(p);
+        *reinterpret_cast<float4*>(t + 4) = *reinterpret_cast<const float4*>(p + 4);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = to_f32(t[e]);
+}
+template <typename T>
+__device__ __forceinline__ void store8(T* p, const T* t) {
+    if (sizeof(T) == 2) {
+        *reinterpret_cast<uint4*>(p) = *reinterpret_cast<const uint4*>(t);
+    } else {
+        *reinterpret_cast<float4*>(p) = *reinterpret_cast<const float4*>(t);
+        *reinterpret_cast<float4*>(p + 4) = *reinterpret_cast<const float4*>(t + 4);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+rope_kvwrite_vec_kernel(T* __restrict__ qkv, const int* __restrict__ pos, const float* __restrict__ cosT,
+                        const float* __restrict__ sinT, T* __restrict__ kc, T* __restrict__ vc,
+                        const int* __restrict__ slots, int nh, int nkv, int d, int rd, int row_stride, int page) {
+    const int t = blockIdx.x;
+    const int half = rd >> 1;
+    const int hp = half >> 3;              // 8-wide pieces of a rotated pair per head
+    const int tail = (d - rd) >> 3;        // 8-wide pieces of a head that are not rotated
+    const int per_qk = hp + tail;          // work items of a q or k head
+    const int per_v = d >> 3;
+    const int slot = slots != nullptr ? slots[t] : -1;
+    const int n_items = (nh + nkv) * per_qk + nkv * per_v;
+    const float* c = cosT + (size_t)pos[t] * half;
+    const float* s = sinT + (size_t)pos[t] * half;
+    T* row = qkv + (size_t)t * row_stride;
+    for (int it = threadIdx.x; it < n_items; it += 256) {
+        if (it < (nh + nkv) * per_qk) {
+            const int hs = it / per_qk, piece = it % per_qk;
+            T* p = row + (size_t)hs * d;
+            T* dst = nullptr;
+            if (hs >= nh && slot >= 0) dst = kc + (((size_t)(slot / page) * nkv + (hs - nh)) * page + (slot % page)) * d;
+            if (piece < hp) {
+                const int i = piece * 8;
+                float a[8], b[8], cc[8], ss[8];
+                load8(p + i, a);
+                load8(p + i + half, b);
+                load8(c + i, cc);
+                load8(s + i, ss);
+                T ra[8], rb[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    ra[e] = from_f32<T>(a[e] * cc[e] - b[e] * ss[e]);
+                    rb[e] = from_f32<T>(b[e] * cc[e] + a[e] * ss[e]);
+                }
+                store8(p + i, ra);
+                store8(p + i + half, rb);
+                if (dst != nullptr) {
+                    store8(dst + i, ra);
+                    store8(dst + i + half, rb);
+                }
+            } else if (dst != nullptr) {
+                const int i = rd + (piece - hp) * 8;
+                T v8[8];
+                store8(v8, p + i);
+                store8(dst + i, v8);
+            }
+        } else if (slot >= 0) {
+            const int j = it - (nh + nkv) * per_qk;
+            const int kvh = j / per_v, i = (j % per_v) * 8;
+            T v8[8];
+            store8(v8, row + (size_t)(nh + nkv + kvh) * d + i);
+            T* vdst = vc + ((size_t)(slot / page) * nkv + kvh) * d * page + (slot % page);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) vdst[(size_t)(i + e) * page] = v8[e];
+        }
+    }
+}
+
 extern "C" int ilm_rope_kvwrite(void* qkv, const void* pos, const void* cosT, const void* sinT,
                                 void* kc, void* vc, const void* slots, int T_, int nh, int nkv,
                                 int d, int rd, int row_stride, int page, int dtype,
@@ -230,6 +313,22 @@ extern "C" int ilm_rope_kvwrite(void* qkv, const void* pos, const void* cosT, co
     ILM_REQUIRE(rd >= 0 && rd <= d && rd % 2 == 0, "rope_kvwrite: rotary dim %d does not fit head dim %d", rd, d);
     ILM_REQUIRE(row_stride >= (nh + 2 * nkv) * d, "rope_kvwrite: row stride %d too small", row_stride);
     ILM_REQUIRE(slots == nullptr || page > 0, "rope_kvwrite: page size %d", page);
+    const bool vec = rd % 16 == 0 && d % 8 == 0 && row_stride % 8 == 0 && ((uintptr_t)qkv & 31) == 0 &&
+                     ((uintptr_t)kc & 31) == 0 && ((uintptr_t)cosT & 31) == 0 && ((uintptr_t)sinT & 31) == 0;
+    if (vec && dtype == ILM_DTYPE_F32) {
+        rope_kvwrite_vec_kernel<float><<<T_, 256, 0, stream>>>((float*)qkv, (const int*)pos, (const float*)cosT,
+                                                              (const float*)sinT, (float*)kc, (float*)vc,
+                                                              (const int*)slots, nh, nkv, d, rd, row_stride, page);
+        ILM_LAUNCH_CHECK("rope_kvwrite");
+        return 0;
+    }
+    if (vec && dtype == ILM_DTYPE_BF16) {
+        rope_kvwrite_vec_kernel<bf16><<<T_, 256, 0, stream>>>((bf16*)qkv, (const int*)pos, (const float*)cosT,
+                                                             (const float*)sinT, (bf16*)kc, (bf16*)vc,
+                                                             (const int*)slots, nh, nkv, d, rd, row_stride, page);
+        ILM_LAUNCH_CHECK("rope_kvwrite");
+        return 0;
+    }
     dim3 grid(T_, nh + 2 * nkv);
     if (dtype == ILM_DTYPE_F32)
         rope_kvwrite_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, (const int*)pos, (const float*)cosT,

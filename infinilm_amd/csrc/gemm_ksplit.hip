@@ -8,6 +8,8 @@
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 
 #define GF_KSPAN 4096   // K a workgroup covers: waves x k-steps x 32
 
@@ -15,7 +17,10 @@ __device__ __forceinline__ f32x4 gf_mfma(uint4 a, uint4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 // 16 waves x 8 k-steps keep a wave under 128 registers (4 waves a SIMD, one workgroup a CU).
-template <int GF_WAVES, int GF_KSTEPS, typename TC>
+// ACT: X holds rows [gate | up] of 2K elements and the fragment is made on the fly,
+// x = silu(gate) * up (the SwiGLU between the two projections of a feed-forward), instead of being
+// read: one kernel and one trip through memory less a layer.
+template <int GF_WAVES, int GF_KSTEPS, bool ACT, typename TC>
 __global__ void __launch_bounds__(GF_WAVES * 64)
 gemm_ksplit_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
                    const bf16* __restrict__ bias, int M, int N, int K, int lda, int ldw, int ldc, float alpha,
@@ -53,7 +58,23 @@ gemm_ksplit_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* _
         const uint4* xp = reinterpret_cast<const uint4*>(X + (size_t)(row_ok ? r : 0) * lda);
 #pragma unroll
         for (int u = 0; u < GF_KSTEPS; ++u) {
-            const uint4 v = xp[k8c[u]];
+            uint4 v = xp[k8c[u]];
+            if (ACT) {
+                const uint4 up = xp[k8c[u] + (K >> 3)];
+                const uint32_t gw[4] = {v.x, v.y, v.z, v.w}, uw[4] = {up.x, up.y, up.z, up.w};
+                uint32_t o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
+                    const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
+                    // hardware exp2 and reciprocal (about 1 ulp each): the result is rounded to bfloat16 anyway
+                    const float s0_ = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g0));
+                    const float s1_ = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g1));
+                    const f32x2 pr = {g0 * s0_ * u0, g1 * s1_ * u1};
+                    o[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf16x2));
+                }
+                v = make_uint4(o[0], o[1], o[2], o[3]);
+            }
             xf[u] = (kok[u] && row_ok) ? v : zero;   // zero fragments make the clamped W loads harmless
         }
     }
@@ -105,31 +126,34 @@ static int gf_num_cus() {
 extern "C" int ilm_gemm_ksplit_max_k(int parts) { return GF_KSPAN * parts; }
 
 // kb > 1: C must be float, [kb][M][ldc] with c_part_stride elements between the parts.
+// act != 0: X rows are [gate | up] (2K long) and the product takes silu(gate) * up.
 extern "C" int ilm_gemm_ksplit(void* C, int out_dtype, int ldc, long c_part_stride, int kb, const void* W, int ldw,
                                const void* bias, float alpha, int M, int N, int K, const void* X, int lda,
-                               hipStream_t stream) {
+                               int act, hipStream_t stream) {
     ILM_REQUIRE(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_ksplit: needs 1 <= M <= 16, got M=%d N=%d K=%d", M, N, K);
     ILM_REQUIRE(K % 8 == 0 && ldw % 8 == 0 && ldw >= K && ldc >= N, "gemm_ksplit: K=%d ldw=%d ldc=%d", K, ldw, ldc);
     ILM_REQUIRE(kb >= 1 && K <= ilm_gemm_ksplit_max_k(kb), "gemm_ksplit: K=%d does not fit %d parts of %d", K, kb,
                 GF_KSPAN);
     ILM_REQUIRE(kb == 1 || out_dtype == ILM_DTYPE_F32, "gemm_ksplit: partial results are float");
-    ILM_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && lda % 8 == 0 && lda >= K,
-                "gemm_ksplit: X and W rows must be 16-byte aligned");
+    ILM_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && lda % 8 == 0 && lda >= (act ? 2 * K : K),
+                "gemm_ksplit: X and W rows must be 16-byte aligned, X rows %d long", act ? 2 * K : K);
     const int ntiles = (N + 15) / 16;
     int gx = gf_num_cus() / kb;
     if (gx < 1) gx = 1;
     if (gx > ntiles) gx = ntiles;
     dim3 grid(gx, kb);
-    if (out_dtype == ILM_DTYPE_BF16)
-        gemm_ksplit_kernel<16, 8, bf16><<<grid, 16 * 64, 0, stream>>>((bf16*)C, (const bf16*)X, (const bf16*)W,
-                                                                      (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha,
-                                                                      ntiles, (size_t)c_part_stride);
-    else if (out_dtype == ILM_DTYPE_F32)
-        gemm_ksplit_kernel<16, 8, float><<<grid, 16 * 64, 0, stream>>>((float*)C, (const bf16*)X, (const bf16*)W,
-                                                                       (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha,
-                                                                       ntiles, (size_t)c_part_stride);
-    else
+#define KS_LAUNCH(ACT, TC)                                                                                     \
+    gemm_ksplit_kernel<16, 8, ACT, TC><<<grid, 16 * 64, 0, stream>>>((TC*)C, (const bf16*)X, (const bf16*)W,   \
+                                                                     (const bf16*)bias, M, N, K, lda, ldw, ldc, \
+                                                                     alpha, ntiles, (size_t)c_part_stride)
+    if (out_dtype == ILM_DTYPE_BF16) {
+        if (act) KS_LAUNCH(true, bf16); else KS_LAUNCH(false, bf16);
+    } else if (out_dtype == ILM_DTYPE_F32) {
+        if (act) KS_LAUNCH(true, float); else KS_LAUNCH(false, float);
+    } else {
         ILM_REQUIRE(false, "gemm_ksplit: unknown output dtype %d", out_dtype);
+    }
+#undef KS_LAUNCH
     ILM_LAUNCH_CHECK("gemm_ksplit");
     return 0;
 }

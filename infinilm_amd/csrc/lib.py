@@ -21,7 +21,7 @@ _L = c_long
 _SIGNATURES = {
     "ilm_embed": [_P, _P, _P, _I, _I, _I, _F, _I, _P],
     "ilm_add_rmsnorm": [_P, _P, _P, _P, _I, _I, _F, _F, _I, _I, _I, _I, _L, _P],
-    "ilm_gemm_ksplit": [_P, _I, _I, _L, _I, _P, _I, _P, _F, _I, _I, _I, _P, _I, _P],
+    "ilm_gemm_ksplit": [_P, _I, _I, _L, _I, _P, _I, _P, _F, _I, _I, _I, _P, _I, _I, _P],
     "ilm_rope_kvwrite": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "ilm_swiglu": [_P, _P, _I, _I, _I, _I, _P],
     "ilm_gather_rows": [_P, _P, _P, _I, _I, _I, _P],

@@ -190,7 +190,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
         kb = -(-K // KSPLIT_SPAN)
         parts = torch.empty((kb, M, N), dtype=F32, device=a.device)
         _run("ilm_gemm_ksplit", parts.data_ptr(), _DT[F32], N, M * N, kb, w.data_ptr(), w.stride(0), None, 1.0,
-             M, N, K, a.data_ptr(), a.stride(0), _stream())
+             M, N, K, a.data_ptr(), a.stride(0), 0, _stream())
         return parts
     if fast and aligned and allow_parts and out is None and M <= 16:
         out_dtype = F32   # a branch on its way into the float32 residual sum need not be rounded first
@@ -211,6 +211,24 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     _run("ilm_gemm_basic", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0), w.stride(0),
          out.stride(0), float(alpha), _dt(a), _DT[out_dtype], _stream())
     return out
+
+
+def swiglu_gemm(gate_up: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
+    """(silu(gate) * up) w^T for at most 16 rows [gate | up] in bfloat16, in one kernel: float32 parts
+    [P, M, N] for add_rmsnorm.  None when the shapes do not fit (the caller then runs the two kernels)."""
+    M, two_k = gate_up.shape
+    K = two_k // 2
+    N = w.shape[0]
+    ok = (gate_up.dtype == BF16 and w.dtype == BF16 and not FORCE_BASIC and USE_KSPLIT and M <= 16 and two_k % 2 == 0
+          and w.shape[1] == K and K % 8 == 0 and gate_up.stride(1) == 1 and w.stride(1) == 1 and gate_up.stride(0) % 8 == 0
+          and w.stride(0) % 8 == 0 and gate_up.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and gate_up.is_cuda)
+    if not ok:
+        return None
+    kb = -(-K // KSPLIT_SPAN)
+    parts = torch.empty((kb, M, N), dtype=F32, device=gate_up.device)
+    _run("ilm_gemm_ksplit", parts.data_ptr(), _DT[F32], N, M * N, kb, w.data_ptr(), w.stride(0), None, 1.0,
+         M, N, K, gate_up.data_ptr(), gate_up.stride(0), 1, _stream())
+    return parts
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,

@@ -28,4 +28,9 @@ class SwiGLU(FeedForward):
         return out
 
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
-        return self.down.forward(kernels.swiglu(self.gate_up.forward(x)), allow_parts=True)
+        gu = self.gate_up.forward(x)
+        if self.down.bias is None:
+            fused = kernels.swiglu_gemm(gu, self.down.weight)   # few rows: activation inside the product
+            if fused is not None:
+                return fused
+        return self.down.forward(kernels.swiglu(gu), allow_parts=True)

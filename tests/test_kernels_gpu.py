@@ -166,6 +166,17 @@ def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
     _close(x, P.plain_rmsnorm(want_r, nw.to(F64), 1e-6), 1e-2)
 
 
+@pytest.mark.parametrize("M,I,N", [(8, 16384, 4096), (3, 200, 96), (16, 4104, 50)])
+def test_swiglu_inside_the_down_projection(K, M, I, N):
+    gu = _rand((M, 2 * I), 18, torch.bfloat16, 1.5)
+    w = _rand((N, I), 19, torch.bfloat16, 0.05)
+    parts = K.swiglu_gemm(gu.to(DEV), w.to(DEV))
+    assert parts is not None and parts.dtype == torch.float32 and parts.shape == (-(-I // 4096), M, N)
+    act = P.plain_swiglu(gu.to(F64)[:, :I], gu.to(F64)[:, I:])
+    _close(parts.sum(0), P.plain_linear(act, w.to(F64)), 6e-3)   # the activation is rounded to bfloat16 once
+    assert K.swiglu_gemm(_rand((17, 64), 1, torch.bfloat16).to(DEV), _rand((8, 32), 2, torch.bfloat16).to(DEV)) is None
+
+
 def _paged(k, v, page, n_pages, seed, dtype):
     """Scatters contiguous per-request keys/values [n, nkv, d] into a paged cache with a shuffled
     block table; unused slots hold large finite garbage so that a read beyond a length shows."""
