@@ -300,3 +300,139 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         err = rel_err(drv.request_logits(r, len(ids)), _toy_plain(cfg, W, ids))
         assert err < 1e-4, f"request {r}: error {err:.3e}"
     assert drv.runner.cache.free_pages() == 24
+
+
+def test_attention_without_rotation_is_the_library_routine():
+    """Position encoding `none`: the mixer reduces to projections around plain causal attention."""
+    import torch.nn.functional as F
+    from infinilm_amd.parts.registry import build_mixer
+    from infinilm_amd.config import PartSpec
+
+    H, nh, nkv, d, n = 48, 4, 4, 16, 40
+    att = build_mixer(PartSpec("gqa_attention", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d,
+                                                 "qkv_bias": False, "out_bias": False, "scale": d ** -0.5, "window": 0,
+                                                 "position": PartSpec("none", {"head_dim": d})}), _ctx(torch.float32))
+    W = _fill(att, 11)
+    hz = _Harness([att.cache_need()], torch.float32, page_size=8, num_pages=8)
+    x = torch.randn(n, H)
+    b = hz.batch([("r", n)])
+    got = att.forward(x.to(DEV), b, hz.cache.view(0, b, True))
+    xd = x.to(F64)
+    q, k, v = (F.linear(xd, W[f"{p}_proj.weight"]).view(n, nh, d).transpose(0, 1) for p in "qkv")
+    o = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(0, 1).reshape(n, nh * d)
+    assert rel_err(got, F.linear(o, W["o_proj.weight"])) < 5e-6
+
+
+def test_a_rope_scaling_registered_from_outside():
+    """Another scaling of the rotary encoding is one registered function; the mixer needs no change."""
+    from infinilm_amd.parts import register_rope_scaling
+    from infinilm_amd.parts.registry import build_position_encoding
+    from infinilm_amd.config import PartSpec
+
+    @register_rope_scaling("toy_linear")
+    def _linear(inv_freq, params, max_positions):
+        return inv_freq / float(params["factor"]), 1.0
+
+    rope = build_position_encoding(PartSpec("rotary", {"head_dim": 32, "rotary_dim": 16, "max_positions": 64, "theta": 100.0,
+                                                       "scaling": {"type": "toy_linear", "factor": 4.0}}), _ctx(torch.float32))
+    i = torch.arange(8, dtype=F64)
+    ang = torch.arange(64, dtype=F64)[:, None] * (1.0 / (4.0 * 100.0 ** (2 * i / 16)))[None, :]
+    assert rel_err(rope.cos, torch.cos(ang)) < 1e-6 and rel_err(rope.sin, torch.sin(ang)) < 1e-6
+
+
+def test_toy_feed_forward_with_routing(tmp_path):
+    """A feed-forward that routes every token to one of three experts, defined and registered here,
+    in a model whose layers use different feed-forwards; portions and batches give the whole-sequence result."""
+    from safetensors.torch import save_file
+    from infinilm_amd import kernels
+    from infinilm_amd.config import HeadSpec, LayerRun, LayerSpec, ModelSpec, PartSpec, register_architecture
+    from infinilm_amd.engine.loading import build_model
+    from infinilm_amd.parts import FeedForward, Param, register_feed_forward
+    from helpers import Driver
+
+    @register_feed_forward("toy_top1_experts")
+    class ToyExperts(FeedForward):
+        def __init__(self, hidden_size, intermediate_size, num_experts, ctx):
+            self.E = int(num_experts)
+            self.router = torch.empty((self.E, hidden_size), dtype=torch.float32, device=ctx.device)
+            self.gate_up = [torch.empty((2 * intermediate_size, hidden_size), dtype=ctx.dtype, device=ctx.device) for _ in range(self.E)]
+            self.down = [torch.empty((hidden_size, intermediate_size), dtype=ctx.dtype, device=ctx.device) for _ in range(self.E)]
+
+        def named_parameters(self):
+            out = {"router.weight": Param(self.router)}
+            for e in range(self.E):
+                out[f"experts.{e}.gate_up.weight"] = Param(self.gate_up[e])
+                out[f"experts.{e}.down.weight"] = Param(self.down[e])
+            return out
+
+        def forward(self, x, batch):
+            choice = kernels.argmax(kernels.gemm(x.float(), self.router)).long()   # router logits in float32
+            out = torch.zeros_like(x)
+            for e in range(self.E):
+                rows = torch.nonzero(choice == e).flatten()
+                if rows.numel():
+                    xe = x.index_select(0, rows).contiguous()
+                    out.index_copy_(0, rows, kernels.gemm(kernels.swiglu(kernels.gemm(xe, self.gate_up[e])), self.down[e]))
+            return out
+
+    def build_spec(cfg):
+        H, d = cfg["hidden_size"], cfg["head_dim"]
+        norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-6})
+        pos = PartSpec("rotary", {"head_dim": d, "rotary_dim": d, "max_positions": 128, "theta": 1e4, "scaling": None})
+        att = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": d, "qkv_bias": False,
+                                         "out_bias": False, "scale": d ** -0.5, "window": 0, "position": pos})
+        dense = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 40, "bias": False})
+        moe = PartSpec("toy_top1_experts", {"hidden_size": H, "intermediate_size": 24, "num_experts": 3})
+        names = {"norm1": "ln1", "mixer": "att", "norm2": "ln2", "ffn": "ffn"}
+        layers = [LayerSpec(f"l.{i}", "pre_norm", {"norm1": norm, "mixer": att, "norm2": norm, "ffn": f}, names, 1.0)
+                  for i, f in enumerate([dense, moe])]
+        return ModelSpec("ToyRoutedLM", cfg["vocab_size"], H, 128, "emb", 1.0, layers, [LayerRun(0, 0), LayerRun(1, 1)], norm,
+                         "ln_f", HeadSpec("head", 1.0, True))
+
+    register_architecture(["ToyRoutedLM"], dict, build_spec)
+    cfg = {"architectures": ["ToyRoutedLM"], "torch_dtype": "float32", "vocab_size": 61, "hidden_size": 32, "head_dim": 16}
+    d = str(tmp_path / "routed")
+    os.makedirs(d)
+    json.dump(cfg, open(os.path.join(d, "config.json"), "w"))
+    g = torch.Generator().manual_seed(8)
+    W = {}
+    for name, p in sorted(build_model(cfg, "float32", "meta").named_parameters().items()):
+        if name == "head.weight":
+            continue
+        t = torch.randn(tuple(p.tensor.shape), generator=g) * 0.4
+        W[name] = (t * 0.25 + 1.0) if t.dim() == 1 else t
+    save_file(W, os.path.join(d, "model.safetensors"), metadata={"format": "pt"})
+
+    def plain(ids):
+        Wd = {k: v.to(F64) for k, v in W.items()}
+        n = len(ids)
+        cos, sin = P.plain_rope_tables({"hidden_size": 16, "num_attention_heads": 1, "max_position_embeddings": 128})
+        pos = torch.arange(n)
+        x = Wd["emb.weight"][torch.tensor(ids)]
+        for l in range(2):
+            p = f"l.{l}."
+            h = P.plain_rmsnorm(x, Wd[p + "ln1.weight"], 1e-6)
+            q = P.plain_apply_rope(P.plain_linear(h, Wd[p + "att.q_proj.weight"]).view(n, 2, 16), pos, cos, sin, 16)
+            k = P.plain_apply_rope(P.plain_linear(h, Wd[p + "att.k_proj.weight"]).view(n, 1, 16), pos, cos, sin, 16)
+            v = P.plain_linear(h, Wd[p + "att.v_proj.weight"]).view(n, 1, 16)
+            x = x + P.plain_linear(P.plain_attention(q, k, v, 0.25).reshape(n, 32), Wd[p + "att.o_proj.weight"])
+            h = P.plain_rmsnorm(x, Wd[p + "ln2.weight"], 1e-6)
+            if l == 0:
+                x = x + P.plain_mlp(h, Wd[p + "ffn.gate_proj.weight"], Wd[p + "ffn.up_proj.weight"], Wd[p + "ffn.down_proj.weight"], 1.0)
+            else:
+                choice = torch.argmax(h @ Wd[p + "ffn.router.weight"].T, dim=-1)
+                y = torch.zeros_like(h)
+                for t in range(n):
+                    gu = Wd[p + f"ffn.experts.{int(choice[t])}.gate_up.weight"]
+                    y[t] = P.plain_mlp(h[t:t + 1], gu[:24], gu[24:], Wd[p + f"ffn.experts.{int(choice[t])}.down.weight"], 1.0)[0]
+                x = x + y
+        return P.plain_linear(P.plain_rmsnorm(x, Wd["ln_f.weight"], 1e-6), Wd["emb.weight"])
+
+    drv = Driver(d, "float32", num_pages=16, page_size=8, max_requests=2)
+    g2 = torch.Generator().manual_seed(3)
+    a, b = (torch.randint(0, 61, (n,), generator=g2).tolist() for n in (45, 20))
+    drv.step([("a", a[:17])])
+    drv.step([("a", a[17:19]), ("b", b)], end=["b"])
+    drv.step([("a", a[19:])], end=["a"])
+    assert rel_err(drv.request_logits("a", 45), plain(a)) < 1e-4
+    assert rel_err(drv.request_logits("b", 20), plain(b)) < 1e-4
