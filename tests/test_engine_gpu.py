@@ -263,3 +263,45 @@ def test_command_line(models):
     want = str(P.plain_greedy(cfg, W, prompt, 7))
     assert proc.stdout.count(want) == 2, proc.stdout[-1500:]
     assert "total_time:" in proc.stdout
+
+
+def test_layers_of_real_size_bfloat16_against_float32():
+    """Two layers of the 8B shape (hidden 4096, 32 heads in 2 groups, head 128, intermediate 16384,
+    vocabulary 73448): the bfloat16 kernels that serving uses at that size (resident and K-split
+    few-rows products, tile and chunked attention over pages of 64, graph replay) against the
+    float32 path on the same weights: a 600-token prompt in portions, then decoded tokens."""
+    from infinilm_amd.engine.loading import build_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+    from infinilm_amd.weights import fill_random_
+
+    cfg = {"architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm", "num_hidden_layers": 2, "hidden_size": 4096,
+           "num_attention_heads": 32, "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 16384,
+           "vocab_size": 73448, "max_position_embeddings": 4096, "rms_norm_eps": 1e-6, "scale_emb": 12, "scale_depth": 1.4,
+           "dim_model_base": 256, "rope_theta": 10000.0,
+           "rope_scaling": {"type": "longrope", "short_factor": [1.0 + i / 64 for i in range(64)],
+                            "long_factor": [2.0] * 64, "original_max_position_embeddings": 4096}}
+    g = torch.Generator().manual_seed(5)
+    prompt = torch.randint(0, 73448, (600,), generator=g).tolist()
+    logits, fed = {}, []
+    for dtype, graph in (("float32", False), ("bfloat16", True)):
+        model = build_model(cfg, dtype, "cuda:0")
+        fill_random_(model, seed=1, std=0.02, norm_init="one_plus")
+        if dtype == "float32":   # the same values the bfloat16 model holds
+            for p in model.named_parameters().values():
+                p.tensor.copy_(p.tensor.to(torch.bfloat16).to(torch.float32))
+        r = make_runner(model, num_pages=16, page_size=64, max_requests=2, enable_graph=graph)
+        r.cache.admit("a")
+        rows = [r.step([StepEntry("a", prompt[:300], [0, 299])]).cpu().clone()]
+        rows.append(r.step([StepEntry("a", prompt[300:599], [298])]).cpu().clone())
+        tok = prompt[599]
+        for i in range(6):
+            l = r.step([StepEntry("a", [tok], [0])]).cpu().clone()
+            rows.append(l)
+            if dtype == "float32":
+                fed.append(int(torch.argmax(l[0])))
+            tok = fed[i]   # both runs are fed the float32 run's greedy tokens
+        logits[dtype] = torch.cat(rows)
+        del r, model
+        torch.cuda.empty_cache()
+    err = rel_err(logits["bfloat16"], logits["float32"])
+    assert err < TOL["bfloat16"], f"bfloat16 against float32 at real size: {err:.3e}"
