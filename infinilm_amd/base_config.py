@@ -9,14 +9,16 @@ from typing import List, Optional
 
 
 class BaseConfig:
-    def __init__(self, argv: Optional[List[str]] = None):
+    def __init__(self, argv: Optional[List[str]] = None, batch_size_type=int):
+        """`batch_size_type=str` lets a benchmark take a list ("1,8,64") where generation takes a number."""
         ap = argparse.ArgumentParser(description="infinilm_amd generation example")
         ap.add_argument("--model", type=str, required=True, help="model directory (config.json + safetensors)")
         ap.add_argument("--device", type=str, default="auto", help="always the AMD GPU; kept for compatibility")
         ap.add_argument("--device-id", type=int, default=0)
         ap.add_argument("--dtype", type=str, default=None, choices=["float32", "bfloat16"],
                         help="overrides config.json's dtype; float32 is true 32-bit throughout")
-        ap.add_argument("--batch-size", type=int, default=1, help="number of copies of the prompt")
+        ap.add_argument("--batch-size", type=batch_size_type, default=batch_size_type(1),
+                        help="number of copies of the prompt")
         ap.add_argument("--prompt", type=str, default="How are you")
         ap.add_argument("--prompt-ids", type=str, default=None,
                         help="comma-separated token ids instead of --prompt (no tokenizer needed)")

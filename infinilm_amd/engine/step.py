@@ -71,6 +71,8 @@ class StepRunner:
         self.enable_graph = bool(enable_graph)
         self._graphs: Dict = {}          # (requests, block-table width) -> (graph, batch, logits, buffer)
         self._graph_pool = None
+        self._graph_seen: Dict = {}      # sizes met in eager steps so far -> how often
+        self.graph_after = 2
         self._pinned: Optional[torch.Tensor] = None
         self._copy_done: Optional[torch.cuda.Event] = None
         self.steps = 0
@@ -246,7 +248,11 @@ class StepRunner:
         a captured HIP graph; the returned tensor is then the graph's output buffer, valid until
         the next such step."""
         if self.enable_graph and taps is None and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-            return self._graph_step(entries)
+            key = self._graph_key(entries)
+            if key not in self._graphs:
+                self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
+            if key in self._graphs or self._graph_seen[key] >= self.graph_after:
+                return self._graph_step(entries, key)
         batch = self.build_batch(entries)
         batch.taps = taps
         logits = self.model.forward(batch, self.cache)
@@ -257,20 +263,25 @@ class StepRunner:
         return logits
 
     # ---- decode steps as captured graphs ----------------------------------------------------------
-    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """One graph per (number of requests, block-table width).  The width is rounded up to a power
-        of two, so a graph serves every context up to width * page tokens; the kernels' grids are
-        sized for that bound and bound their reads by each request's own length.  Between replays
-        only the metadata buffer changes (token ids, positions, slots, block tables).
-        Reference: csrc/engine/compiler/paged_compiler.cpp:59-260 (one graph per decode batch size,
-        inputs copied into captured buffers)."""
+    def _graph_key(self, entries: Sequence[StepEntry]):
         cache = self.cache
-        R = len(entries)
         need = max(-(-(cache.length(e.req_id) + 1) // cache.page_size) for e in entries)
         width = 4
         while width < need:
             width *= 2
-        key = (R, width)
+        return (len(entries), width)
+
+    def _graph_step(self, entries: Sequence[StepEntry], key) -> torch.Tensor:
+        """One graph per (number of requests, block-table width).  The width is rounded up to a power
+        of two, so a graph serves every context up to width * page tokens; the kernels' grids are
+        sized for that bound and bound their reads by each request's own length.  Between replays
+        only the metadata buffer changes (token ids, positions, slots, block tables).  A size is
+        recorded the `graph_after`-th time it comes (a recording costs about three steps, which a
+        batch size that passes once, while requests trickle in or out, never earns back).
+        Reference: csrc/engine/compiler/paged_compiler.cpp:59-260 (one graph per decode batch size,
+        inputs copied into captured buffers)."""
+        cache = self.cache
+        R, width = key
         slot = self._graphs.get(key)
         if slot is None:
             buf = torch.zeros((self._graph_buffer_size(R, width),), dtype=torch.int32, device=self.device)

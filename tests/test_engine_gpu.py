@@ -265,6 +265,19 @@ def test_command_line(models):
     assert "total_time:" in proc.stdout
 
 
+def test_benchmark_example(models):
+    """examples/bench.py: the case grid in order of cache size, one JSON line a case."""
+    import json
+    cfg, d, W = models[("B", "bfloat16")]
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "examples", "bench.py"), "--model", d, "--batch-size", "3,1",
+                           "--input-len", "40,7", "--output-len", "5", "--block-size", "16", "--enable-graph", "--warmup"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    rows = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("{")]
+    assert [(r["batch_size"], r["input_len"]) for r in rows] == [(1, 7), (3, 7), (1, 40), (3, 40)]
+    assert all("error" not in r and r["decode_tok_s"] > 0 and r["ttft_ms"] > 0 for r in rows)
+
+
 def test_layers_of_real_size_bfloat16_against_float32():
     """Two layers of the 8B shape (hidden 4096, 32 heads in 2 groups, head 128, intermediate 16384,
     vocabulary 73448): the bfloat16 kernels that serving uses at that size (resident and K-split
