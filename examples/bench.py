@@ -37,9 +37,10 @@ def test_cases(cfg_json: dict, batch_sizes, input_lens, output_lens):
     for b in batch_sizes:
         for i in input_lens:
             for o in output_lens:
-                cases.append({"batch_size": b, "input_len": i, "output_len": o,
-                              "kvcache_gb": round(2 * 2 * b * (i + o) * nkv * d * layers / 2 ** 30, 3)})
-    return sorted(cases, key=lambda c: c["kvcache_gb"])
+                nbytes = 2 * 2 * b * (i + o) * nkv * d * layers
+                cases.append((nbytes, {"batch_size": b, "input_len": i, "output_len": o,
+                                       "kvcache_gb": round(nbytes / 2 ** 30, 3)}))
+    return [c for _, c in sorted(cases, key=lambda nc: nc[0])]
 
 
 def run_case(llm: LLM, case: dict, seed: int, sp_kwargs: dict) -> dict:

@@ -278,27 +278,42 @@ def test_benchmark_example(models):
     assert all("error" not in r and r["decode_tok_s"] > 0 and r["ttft_ms"] > 0 for r in rows)
 
 
-def test_layers_of_real_size_bfloat16_against_float32():
-    """Two layers of the 8B shape (hidden 4096, 32 heads in 2 groups, head 128, intermediate 16384,
-    vocabulary 73448): the bfloat16 kernels that serving uses at that size (resident and K-split
-    few-rows products, tile and chunked attention over pages of 64, graph replay) against the
-    float32 path on the same weights: a 600-token prompt in portions, then decoded tokens."""
+def _real_shape(name):
+    base = {"architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm", "num_hidden_layers": 2, "scale_emb": 12,
+            "scale_depth": 1.4, "dim_model_base": 256, "rope_theta": 10000.0, "max_position_embeddings": 4096}
+    if name == "8b":      # 32 heads in 2 groups of 16, head 128, untied head
+        return dict(base, hidden_size=4096, num_attention_heads=32, num_key_value_heads=2, head_dim=128,
+                    intermediate_size=16384, vocab_size=73448, rms_norm_eps=1e-6,
+                    rope_scaling={"type": "longrope", "short_factor": [1.0 + i / 64 for i in range(64)],
+                                  "long_factor": [2.0] * 64, "original_max_position_embeddings": 4096})
+    if name == "0.5b":    # head 64, 16 heads in 2 groups of 8, tied head
+        return dict(base, hidden_size=1024, num_attention_heads=16, num_key_value_heads=2, head_dim=64,
+                    intermediate_size=4096, vocab_size=73448, rms_norm_eps=1e-6, tie_word_embeddings=True,
+                    rope_scaling={"type": "longrope", "short_factor": [1.0 + i / 32 for i in range(32)],
+                                  "long_factor": [3.0] * 32, "original_max_position_embeddings": 4096})
+    if name == "2b":      # every head its own keys (36 of 64), widths that are no power of two, odd vocabulary
+        return dict(base, hidden_size=2304, num_attention_heads=36, num_key_value_heads=36, head_dim=64,
+                    intermediate_size=5760, vocab_size=122753, rms_norm_eps=1e-5, tie_word_embeddings=True)
+    raise KeyError(name)
+
+
+@pytest.mark.parametrize("shape", ["8b", "0.5b", "2b"])
+def test_layers_of_real_size_bfloat16_against_float32(shape):
+    """Two layers of a real shape (the 8B, the 0.5B and the 2B-family sizes): the bfloat16 kernels
+    that serving uses at that size (resident and K-split few-rows products, tile and chunked
+    attention over pages of 64, graph replay) against the float32 path on the same weights: a
+    600-token prompt in portions, then decoded tokens."""
     from infinilm_amd.engine.loading import build_model, make_runner
     from infinilm_amd.engine.step import StepEntry
     from infinilm_amd.weights import fill_random_
 
-    cfg = {"architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm", "num_hidden_layers": 2, "hidden_size": 4096,
-           "num_attention_heads": 32, "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 16384,
-           "vocab_size": 73448, "max_position_embeddings": 4096, "rms_norm_eps": 1e-6, "scale_emb": 12, "scale_depth": 1.4,
-           "dim_model_base": 256, "rope_theta": 10000.0,
-           "rope_scaling": {"type": "longrope", "short_factor": [1.0 + i / 64 for i in range(64)],
-                            "long_factor": [2.0] * 64, "original_max_position_embeddings": 4096}}
+    cfg = _real_shape(shape)
     g = torch.Generator().manual_seed(5)
-    prompt = torch.randint(0, 73448, (600,), generator=g).tolist()
+    prompt = torch.randint(0, cfg["vocab_size"], (600,), generator=g).tolist()
     logits, fed = {}, []
     for dtype, graph in (("float32", False), ("bfloat16", True)):
         model = build_model(cfg, dtype, "cuda:0")
-        fill_random_(model, seed=1, std=0.02, norm_init="one_plus")
+        fill_random_(model, seed=1, std=0.02, norm_init="one_plus", tie=bool(cfg.get("tie_word_embeddings")))
         if dtype == "float32":   # the same values the bfloat16 model holds
             for p in model.named_parameters().values():
                 p.tensor.copy_(p.tensor.to(torch.bfloat16).to(torch.float32))
