@@ -292,6 +292,14 @@ attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, cons
 #define ATT_NT 2
 #define ATT_TK 64        // keys per tile
 #define ATT_BT_LDS 2048  // block-table entries kept in LDS
+#define ATT_LAZY 8.0f    // the exponent's reference point follows the maximum in steps of at least this
+
+// maximum of three without the quieting of NaN that fmaxf brings (scores are finite)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float d;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
 
 template <int D16, bool PAGE64>
 __global__ void __launch_bounds__(256, 2)
@@ -308,10 +316,11 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     __shared__ int bt_s[ATT_BT_LDS];
     // the longest tiles (latest positions) are dispatched first
     const int tile_id = gridDim.x - 1 - blockIdx.x;
+    const int by = blockIdx.y;
     const int t0 = tiles[2 * tile_id], ntok = tiles[2 * tile_id + 1];
     const int G = nh / nkv;
     const int HG = (G + 15) / 16;
-    const int kvh = blockIdx.y / HG, hg = blockIdx.y % HG;
+    const int kvh = by / HG, hg = by % HG;
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, qg = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: what depends on it stays in SGPRs
     const int hcol = hg * 16 + r;
@@ -348,12 +357,13 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
             qf[j][ks] = dofs < D ? v : zero4;
         }
     }
-    f32x4 acc[ATT_NT][D16];
-    float m[ATT_NT], lsum[ATT_NT];
+    f32x4 acc[ATT_NT][D16], lacc[ATT_NT];   // lacc: every element holds the column's sum of p
+    float mc[ATT_NT];                        // reference point of the exponent: (a past maximum) * scale * log2(e)
+    const uint4 ones4 = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);   // bfloat16 1.0
 #pragma unroll
     for (int j = 0; j < ATT_NT; ++j) {
-        m[j] = NEG_BIG;
-        lsum[j] = 0.f;
+        mc[j] = NEG_BIG;
+        lacc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int db = 0; db < D16; ++db) acc[j][db] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -396,7 +406,12 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     };
     auto stash_k = [&](int i, uint4 v) {
         const int pc = tid + i * 256;
-        if (pc < KPIECES) *reinterpret_cast<uint4*>(&Ks[pc / (D / 8)][(pc % (D / 8)) * 8]) = v;
+        // Key kk of the tile lies in row (kk&32) | (kk&4)<<2 | (kk&24)>>1 | (kk&3): the 16 keys that one
+        // score product's lanes read (8 consecutive keys a lane group, two products) are 16
+        // consecutive rows, which the row padding spreads over all banks.
+        const int kk = pc / (D / 8);
+        const int prow = (kk & 32) | ((kk & 4) << 2) | ((kk & 24) >> 1) | (kk & 3);
+        if (pc < KPIECES) *reinterpret_cast<uint4*>(&Ks[prow][(pc % (D / 8)) * 8]) = v;
     };
     auto stash_v = [&](int i, uint4 v) {
         const int pc = tid + i * 256;
@@ -435,17 +450,20 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
         ATT_STASH()
         __syncthreads();
         if (kb + ATT_TK <= p_last) { ATT_FETCH(kb + ATT_TK) }   // in flight while this tile is multiplied
+        // The score products of both 32-key sub-tiles are issued first, so that the matrix cores
+        // work on the second while the vector units do the softmax of the first.
+        constexpr int NSUB = ATT_TK / 32;
+        bool any[NSUB];
+        f32x4 s[NSUB][ATT_NT][2];
 #pragma unroll
-        for (int sub = 0; sub < ATT_TK / 32; ++sub) {
+        for (int sub = 0; sub < NSUB; ++sub) {
             const int kbs = kb + sub * 32;
-            const bool any = kbs <= pj[ATT_NT - 1] && kbs + 32 > loj[0];   // wave-uniform
-            if (!any) continue;
-            // four independent accumulator chains (2 key tiles x 2 tokens), interleaved over d
-            f32x4 s[ATT_NT][2];
+            any[sub] = kbs <= pj[ATT_NT - 1] && kbs + 32 > loj[0];   // wave-uniform
+            if (!any[sub]) continue;
             uint4 kf[2][KS];
 #pragma unroll
             for (int tau = 0; tau < 2; ++tau) {
-                const int row = sub * 32 + (r >> 2) * 8 + tau * 4 + (r & 3);
+                const int row = sub * 32 + tau * 16 + r;   // = key sub*32 + (r>>2)*8 + tau*4 + (r&3)
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     const int dofs = ks * 32 + qg * 8;
@@ -454,73 +472,78 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
                                       : zero4;
                 }
 #pragma unroll
-                for (int j = 0; j < ATT_NT; ++j) s[j][tau] = f32x4{0.f, 0.f, 0.f, 0.f};
+                for (int j = 0; j < ATT_NT; ++j) s[sub][j][tau] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
+            // four independent accumulator chains (2 key tiles x 2 tokens), interleaved over d
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                 for (int tau = 0; tau < 2; ++tau)
 #pragma unroll
-                    for (int j = 0; j < ATT_NT; ++j) s[j][tau] = mfma16(kf[tau][ks], qf[j][ks], s[j][tau]);
-            // Softmax on raw scores: the scale enters the exponent's multiply-add.  Sub-tiles that
-            // every token of the wave sees whole (all but those on the diagonal or a window's edge)
-            // skip the masks, and the accumulators are rescaled only when some row's maximum moved.
-            uint4 pf[ATT_NT];
-            float corr[ATT_NT];
+                    for (int j = 0; j < ATT_NT; ++j) s[sub][j][tau] = mfma16(kf[tau][ks], qf[j][ks], s[sub][j][tau]);
+        }
+#pragma unroll
+        for (int sub = 0; sub < NSUB; ++sub) {
+            if (!any[sub]) continue;
+            const int kbs = kb + sub * 32;
+            // Softmax on raw scores, the scale inside the exponent's multiply-add.  The reference
+            // point mc (in units of the exponent) is not the running maximum itself: it is raised
+            // to a column's maximum only when that exceeds it by more than ATT_LAZY, so p <= 2^ATT_LAZY
+            // and on most sub-tiles no lane talks to another.  The row sums come out of the matrix
+            // cores with the values (a row of ones), from the same rounded p.  Sub-tiles that every
+            // token of the wave sees whole (all but the diagonal and a window's edge) skip the masks.
             const bool full = kbs + 31 <= pj[0] && kbs >= loj[ATT_NT - 1];   // wave-uniform
-            bool moved = false;
+            float sv[ATT_NT][8], lm[ATT_NT];
+            bool over = false;
 #pragma unroll
             for (int j = 0; j < ATT_NT; ++j) {
-                float sv[8];
 #pragma unroll
                 for (int tau = 0; tau < 2; ++tau)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) sv[tau * 4 + e] = s[j][tau][e];
+                    for (int e = 0; e < 4; ++e) sv[j][tau * 4 + e] = s[sub][j][tau][e];
                 if (!full) {
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
                         const int key = kbs + qg * 8 + i;
-                        sv[i] = (key >= loj[j] && key <= pj[j]) ? sv[i] : NEG_BIG;
+                        sv[j][i] = (key >= loj[j] && key <= pj[j]) ? sv[j][i] : NEG_BIG;
                     }
                 }
-                float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float m_new = fmaxf(m[j], mx);
-                corr[j] = (m_new > m[j]) ? __builtin_amdgcn_exp2f((m[j] - m_new) * scale_log2e) : 1.0f;
-                moved = moved || (m_new > m[j]);
-                const float mc = m_new * scale_log2e;
+                lm[j] = max3(max3(sv[j][0], sv[j][1], sv[j][2]), max3(sv[j][3], sv[j][4], sv[j][5]), max3(sv[j][6], sv[j][7], sv[j][7]));
+                over = over || fmaf(lm[j], scale_log2e, -mc[j]) > ATT_LAZY;
+            }
+            if (__builtin_amdgcn_ballot_w64(over) != 0ull) {
+#pragma unroll
+                for (int j = 0; j < ATT_NT; ++j) {
+                    float mx = lm[j];
+                    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                    const float mxc = mx * scale_log2e;
+                    const bool up = mxc - mc[j] > ATT_LAZY;   // the same in the four lanes of a column
+                    const float corr = up ? __builtin_amdgcn_exp2f(mc[j] - mxc) : 1.0f;
+                    mc[j] = up ? mxc : mc[j];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) lacc[j][e] *= corr;
+#pragma unroll
+                    for (int db = 0; db < D16; ++db)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[j][db][e] *= corr;
+                }
+            }
+            uint4 pf[ATT_NT];
+#pragma unroll
+            for (int j = 0; j < ATT_NT; ++j) {
                 float pe[8];
-                float rs = 0.f;
-                if (full) {
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        pe[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, -mc));
-                        rs += pe[i];
-                    }
-                } else {
+                for (int i = 0; i < 8; ++i) pe[i] = __builtin_amdgcn_exp2f(fmaf(sv[j][i], scale_log2e, -mc[j]));
+                if (!full) {   // a masked score of a row that has seen no key yet would give 2^0
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        pe[i] = (sv[i] > 0.5f * NEG_BIG) ? __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, -mc)) : 0.f;
-                        rs += pe[i];
-                    }
+                    for (int i = 0; i < 8; ++i) pe[i] = (sv[j][i] > 0.5f * NEG_BIG) ? pe[i] : 0.f;
                 }
-                rs += __shfl_xor(rs, 16, 64);
-                rs += __shfl_xor(rs, 32, 64);
-                lsum[j] = lsum[j] * corr[j] + rs;
-                m[j] = m_new;
                 pf[j].x = pack_bf16x2(pe[0], pe[1]);
                 pf[j].y = pack_bf16x2(pe[2], pe[3]);
                 pf[j].z = pack_bf16x2(pe[4], pe[5]);
                 pf[j].w = pack_bf16x2(pe[6], pe[7]);
-            }
-            if (__builtin_amdgcn_ballot_w64(moved) != 0ull) {
-#pragma unroll
-                for (int j = 0; j < ATT_NT; ++j)
-#pragma unroll
-                    for (int db = 0; db < D16; ++db)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[j][db][e] *= corr[j];
+                lacc[j] = mfma16(ones4, pf[j], lacc[j]);
             }
             const int key0 = kbs + qg * 8;
             const bool vok = key0 <= p_last && key0 + 8 > lo_first;   // else the tile holds another group's values
@@ -537,7 +560,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
 #pragma unroll
     for (int j = 0; j < ATT_NT; ++j) {
         if (!tok_ok[j]) continue;
-        const float inv = 1.0f / lsum[j];
+        const float inv = 1.0f / lacc[j][0];
         bf16* orow = out + (size_t)tok[j] * out_stride + (size_t)head * D;
 #pragma unroll
         for (int db = 0; db < D16; ++db) {

@@ -200,7 +200,7 @@ def _paged(k, v, page, n_pages, seed, dtype):
     return kc, vc, bt
 
 
-def _attention_case(K, dtype, nh, nkv, d, page, lens, qlens, window=0, seed=0, spike=False):
+def _attention_case(K, dtype, nh, nkv, d, page, lens, qlens, window=0, seed=0, spike=False, ramp=0.0):
     """Requests with `lens[i]` cached keys of which the last `qlens[i]` are this step's queries."""
     ks = [_rand((n, nkv, d), seed + 10 * i + 1, dtype) for i, n in enumerate(lens)]
     vs = [_rand((n, nkv, d), seed + 10 * i + 2, dtype) for i, n in enumerate(lens)]
@@ -210,6 +210,13 @@ def _attention_case(K, dtype, nh, nkv, d, page, lens, qlens, window=0, seed=0, s
         for q, k in zip(qs, ks):
             far = 3 if k.shape[0] > 3 else 0
             k[far] = (q[-1, 0:1, :].float() * 4.0 / math.sqrt(d)).to(dtype)
+    if ramp:
+        # scores of the last query's first head rise by `ramp` (natural units) a key: the running
+        # maximum moves in every tile, by little or by much
+        for q, k in zip(qs, ks):
+            u = q[-1, 0, :].float()
+            u = u / (u @ u)
+            k[:, 0, :] = (k[:, 0, :].float() + torch.arange(k.shape[0])[:, None] * (ramp * math.sqrt(d)) * u).to(dtype)
     n_pages = sum(-(-n // page) for n in lens) + 3
     kc, vc, bt = _paged(ks, vs, page, n_pages, seed, dtype)
     q_rows, seg, pos = [], [], []
@@ -264,6 +271,15 @@ def test_attention_bfloat16_matrix_cores(K, nh, nkv, d, page):
     _close(out, want, 1.2e-2)
     # a far key among hundreds must dominate
     out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[520, 65], qlens=[1, 1], seed=9, spike=True)
+    _close(out, want, 1.2e-2)
+
+
+@pytest.mark.parametrize("ramp", [0.02, 0.7, -0.05])
+def test_attention_bfloat16_with_a_moving_maximum(K, ramp):
+    """The tile kernel moves its exponent's reference point lazily: rising and falling scores."""
+    out, want = _attention_case(K, torch.bfloat16, 32, 2, 128, 64, lens=[700, 130], qlens=[300, 130], seed=11, ramp=ramp)
+    _close(out, want, 1.2e-2)
+    out, want = _attention_case(K, torch.bfloat16, 6, 3, 48, 16, lens=[500, 9], qlens=[77, 9], seed=12, ramp=ramp, window=200)
     _close(out, want, 1.2e-2)
 
 
