@@ -3,6 +3,7 @@
 from __future__ import annotations
 
 import itertools
+import time
 from typing import Dict, List, Optional, Sequence
 
 import torch
@@ -27,6 +28,8 @@ class LLMEngine:
         self.tokenizer = tokenizer
         self._ids = itertools.count()
         self.requests: Dict[str, InferenceRequest] = {}
+        self.counters = {"steps": 0, "prompt_tokens": 0, "generated_tokens": 0, "schedule_s": 0.0, "step_s": 0.0,
+                         "sample_s": 0.0, "update_s": 0.0}
 
     def add_request(self, prompt_token_ids: Sequence[int], sampling_params: Optional[SamplingParams] = None,
                     request_id: Optional[str] = None, prompt: Optional[str] = None) -> InferenceRequest:
@@ -50,7 +53,10 @@ class LLMEngine:
     def step(self) -> List[InferenceRequest]:
         """One step of the step function for whatever the scheduler picks; returns the requests
         that finished in it."""
+        t0 = time.perf_counter()
         out = self.scheduler.schedule()
+        t1 = time.perf_counter()
+        self.counters["schedule_s"] += t1 - t0
         if not out.entries:
             if self.scheduler.waiting and not self.scheduler.running:
                 req = self.scheduler.waiting.popleft()
@@ -62,16 +68,33 @@ class LLMEngine:
             toks = e.request.all_token_ids()[e.start:e.start + e.num_tokens]
             entries.append(StepEntry(e.request.request_id, toks, [e.num_tokens - 1] if e.samples else []))
         logits = self.runner.step(entries)
+        t2 = time.perf_counter()
         samplers = [(e.request.sampling_params, e.request.key, e.request.get_num_generated_tokens())
                     for e in out.entries if e.samples]
-        tokens = self.sampler.sample(logits, samplers)
+        tokens = self.sampler.sample(logits, samplers)   # brings the tokens to the host: waits for the step
+        t3 = time.perf_counter()
         sampled = {e.request.request_id: t for e, t in zip((e for e in out.entries if e.samples), tokens)}
         done = self.scheduler.update(out, sampled)
+        c = self.counters
+        c["steps"] += 1
+        c["prompt_tokens"] += sum(e.num_tokens for e in out.entries if e.start < e.request.get_prompt_length())
+        c["generated_tokens"] += len(tokens)
+        c["step_s"] += t2 - t1
+        c["sample_s"] += t3 - t2
+        c["update_s"] += time.perf_counter() - t3
         if self.tokenizer is not None:
             for e in out.entries:
                 if e.samples:
                     self._detokenize(e.request)
         return done
+
+    def stats(self) -> dict:
+        """Counters of the loop (steps, tokens run, host seconds spent scheduling, launching the step,
+        sampling including the wait for the device, updating) and the scheduler's view of the cache
+        (python/infinilm/llm/scheduler.py:579-598 for the latter)."""
+        out = dict(self.counters)
+        out["cache"] = self.scheduler.get_cache_stats()
+        return out
 
     def _detokenize(self, req: InferenceRequest) -> None:
         text = self.tokenizer.decode(req.output_token_ids, skip_special_tokens=True)

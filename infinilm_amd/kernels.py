@@ -34,8 +34,62 @@ def _lib():
     return _libmod.load()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """The current HIP stream's handle (the raw lookup costs a tenth of `torch.cuda.current_stream()`,
+    which matters with some hundred launches a step)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
+
+
+# ---- timers per kernel entry point, off unless asked for ------------------------------------------
+_TIMES: Optional[dict] = {} if os.environ.get("INFINILM_AMD_KERNEL_TIMES", "0") == "1" else None
+
+
+def enable_timing(on: bool = True) -> None:
+    """Brackets every launch with a pair of events (also: INFINILM_AMD_KERNEL_TIMES=1).  Launches
+    inside a graph capture are not timed.  Costs host time; for looking at a step, not for serving."""
+    global _TIMES
+    _TIMES = {} if on else None
+
+
+def timing_report(reset: bool = True) -> dict:
+    """{entry point: {"calls", "total_ms", "mean_us"}}, after waiting for the device."""
+    if _TIMES is None:
+        return {}
+    torch.cuda.synchronize()
+    out = {}
+    for name, pairs in _TIMES.items():
+        total = sum(a.elapsed_time(b) for a, b in pairs)
+        out[name] = {"calls": len(pairs), "total_ms": round(total, 4), "mean_us": round(1e3 * total / max(len(pairs), 1), 2)}
+    if reset:
+        _TIMES.clear()
+    return dict(sorted(out.items(), key=lambda kv: -kv[1]["total_ms"]))
+
+
+class _timed:
+    """Context of one launch; a no-op when timing is off or the stream is being captured."""
+    __slots__ = ("name", "start")
+
+    def __init__(self, name: str):
+        self.name = name
+        self.start = None
+
+    def __enter__(self):
+        if _TIMES is not None and not torch.cuda.is_current_stream_capturing():
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+        return self
+
+    def __exit__(self, *exc):
+        if self.start is not None:
+            end = torch.cuda.Event(enable_timing=True)
+            end.record()
+            _TIMES.setdefault(self.name, []).append((self.start, end))
+        return False
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -52,7 +106,11 @@ def _dev(*ts: Optional[torch.Tensor]) -> None:
 
 
 def _run(name: str, *args) -> None:
-    rc = getattr(_lib(), name)(*args)
+    if _TIMES is None:
+        rc = getattr(_lib(), name)(*args)
+    else:
+        with _timed(name):
+            rc = getattr(_lib(), name)(*args)
     if rc != 0:
         raise KernelError(_libmod.last_error())
 
@@ -206,7 +264,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     if M > 16 and library_ok:
         # large products go to the vendor library, as the reference's linear layers do
         # (csrc/layers/quantization/none_quantization.cpp:26-46 calls its library's linear)
-        torch.matmul(a, w.t(), out=out)
+        with _timed("library_gemm"):
+            torch.matmul(a, w.t(), out=out)
         return out
     _run("ilm_gemm_basic", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0), w.stride(0),
          out.stride(0), float(alpha), _dt(a), _DT[out_dtype], _stream())

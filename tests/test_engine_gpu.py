@@ -265,6 +265,31 @@ def test_command_line(models):
     assert "total_time:" in proc.stdout
 
 
+def test_kernel_timers_and_engine_counters(models):
+    """The per-entry-point timers behind a flag, and the loop's counters."""
+    from infinilm_amd import LLM, SamplingParams, kernels
+
+    cfg, d, W = models[("A", "bfloat16")]
+    llm = LLM(d, dtype="bfloat16", num_blocks=16, block_size=16, max_batch_size=2)
+    kernels.enable_timing(True)
+    try:
+        prompts = [random_tokens(cfg, 9, 1), random_tokens(cfg, 20, 2)]
+        llm.generate(prompt_token_ids=prompts, sampling_params=SamplingParams(max_tokens=5, top_k=1, ignore_eos=True))
+        rep = kernels.timing_report()
+    finally:
+        kernels.enable_timing(False)
+    L = cfg["num_hidden_layers"]
+    assert rep["ilm_embed"]["calls"] == 5                       # one step of prompts, four of decoded tokens
+    assert rep["ilm_rope_kvwrite"]["calls"] == 5 * L
+    assert rep["ilm_add_rmsnorm"]["calls"] == 5 * (2 * L + 1)
+    assert all(v["total_ms"] > 0 for v in rep.values())
+    assert kernels.timing_report() == {}                        # switched off again
+    st = llm.engine.stats()
+    assert st["steps"] == 5 and st["prompt_tokens"] == 29 and st["generated_tokens"] == 10
+    assert st["cache"]["running"] == 0 and st["cache"]["groups"][0]["free"] == 16
+    llm.close()
+
+
 def test_benchmark_example(models):
     """examples/bench.py: the case grid in order of cache size, one JSON line a case."""
     import json
