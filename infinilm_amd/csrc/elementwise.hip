@@ -434,3 +434,20 @@ extern "C" int ilm_gather_rows(void* out, const void* in, const void* idx, int n
     ILM_LAUNCH_CHECK("gather_rows");
     return 0;
 }
+
+// ------------------------------------------------------------------------------------------
+// x[i, :n] *= alpha over rows of float (the output head's scale after a library product)
+// ------------------------------------------------------------------------------------------
+__global__ void scale_rows_kernel(float* __restrict__ x, int cols, int stride, float alpha) {
+    float* row = x + (size_t)blockIdx.y * stride;
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j < cols) row[j] *= alpha;
+}
+
+extern "C" int ilm_scale_rows(void* x, int rows, int cols, int stride, float alpha, hipStream_t stream) {
+    ILM_REQUIRE(rows > 0 && rows <= 65535 && cols > 0 && stride >= cols, "scale_rows: bad sizes rows=%d cols=%d stride=%d",
+                rows, cols, stride);
+    scale_rows_kernel<<<dim3((cols + 255) / 256, rows), 256, 0, stream>>>((float*)x, cols, stride, alpha);
+    ILM_LAUNCH_CHECK("scale_rows");
+    return 0;
+}

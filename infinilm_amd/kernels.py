@@ -217,6 +217,7 @@ def gather_rows(x: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
     return out
 
 
+_LIBRARY_F32_OUT = [True]   # cleared when torch.mm refuses out_dtype
 KSPLIT_SPAN = 4096  # K range of one part of the K-split few-rows product (ilm_gemm_ksplit_max_k(1))
 
 
@@ -257,6 +258,20 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     library_ok = fast and plain and out_dtype == BF16 and USE_LIBRARY_GEMM
     # measured at the 8B shapes: the few-rows kernel beats the vendor library up to 16 rows and loses
     # to it above (its X fragments are re-read from L2 for every 16 rows of W)
+    if (M > 16 and fast and bias is None and out_dtype == F32 and USE_LIBRARY_GEMM and _LIBRARY_F32_OUT[0]
+            and M <= 65535):
+        # bfloat16 operands, float32 accumulation and result (the output head with many rows)
+        try:
+            with _timed("library_gemm"):
+                torch.mm(a, w.t(), out_dtype=F32, out=out)
+        except (TypeError, RuntimeError) as exc:
+            if "out_dtype" not in str(exc):
+                raise
+            _LIBRARY_F32_OUT[0] = False   # this build of the library door has no float32 result
+        else:
+            if alpha != 1.0:
+                _run("ilm_scale_rows", out.data_ptr(), M, N, out.stride(0), float(alpha), _stream())
+            return out
     if fast and aligned and M <= 64 and not (M > 16 and library_ok):
         _run("ilm_gemm_skinny", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
              w.stride(0), out.stride(0), float(alpha), _DT[out_dtype], SKINNY_VARIANT, _stream())

@@ -129,11 +129,11 @@ def test_gemm_float32_is_true_float32(K, M, N, K_):
     (1, 16, 32, torch.bfloat16), (1, 4608, 4096, torch.bfloat16), (8, 331, 80, torch.float32), (17, 96, 200, torch.bfloat16),
     (33, 200, 96, torch.bfloat16), (64, 73448, 128, torch.float32), (48, 100, 2048, torch.bfloat16),
     (7, 50, 100, torch.bfloat16),        # K no multiple of 8: the plain kernel takes it
-    (100, 176, 80, torch.bfloat16), (300, 512, 256, torch.bfloat16), (65, 40, 64, torch.float32),
+    (100, 176, 80, torch.bfloat16), (300, 512, 256, torch.bfloat16), (65, 40, 64, torch.float32), (40, 331, 96, torch.float32),
 ])
 def test_gemm_bfloat16(K, M, N, K_, out_dtype):
     a, w = _rand((M, K_), 11, torch.bfloat16), _rand((N, K_), 12, torch.bfloat16)
-    alpha = 0.5 if out_dtype == torch.float32 else 1.0
+    alpha = 0.3 if out_dtype == torch.float32 else 1.0
     out = K.gemm(a.to(DEV), w.to(DEV), None, alpha, out_dtype)
     assert out.dtype == out_dtype
     want = P.plain_linear(a.to(F64), w.to(F64), None, alpha)
