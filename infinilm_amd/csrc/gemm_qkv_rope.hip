@@ -1,0 +1,165 @@
+// The fused q/k/v projection of a decode step (at most 16 rows of X, bfloat16) with the rotation of
+// q and k and the write of k and v into the paged cache in its epilogue: one kernel instead of
+// two between the norm and the attention.
+//
+// The product is the resident few-rows one (X fragments in registers, W streamed once on
+// v_mfma_f32_16x16x32_bf16, K split over the waves and reduced through LDS).  A workgroup takes
+// units of two 16-row tiles of W, rows [hs*d + j*16, +16) and [hs*d + d/2 + j*16, +16) of head slot
+// hs: the two halves of 16 rotation pairs.  The thread that reduces output (m, n) of the first
+// tile also reduces (m, n) of the second, so it holds a pair in registers, rotates it by the
+// token's position and stores it: q into the output rows, k into the token's cache slot; v tiles
+// take the same path without rotation into the transposed value cache.
+// Needs the whole head rotated (rotary dim = head dim) and head dims in steps of 32.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__device__ __forceinline__ f32x4 qr_mfma(uint4 a, uint4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// round to bfloat16 and back: the unfused path stores the projection in bfloat16 before it rotates
+__device__ __forceinline__ float qr_round(float v) { return to_f32(from_f32<bf16>(v)); }
+
+template <int WAVES, int KSTEPS>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_qkv_rope_kernel(bf16* __restrict__ Q, const bf16* __restrict__ X, const bf16* __restrict__ W,
+                     const bf16* __restrict__ bias, int M, int K, int lda, int ldw, int ldq,
+                     const int* __restrict__ pos, const float* __restrict__ cosT, const float* __restrict__ sinT,
+                     bf16* __restrict__ kc, bf16* __restrict__ vc, const int* __restrict__ slots, int nh, int nkv,
+                     int d, int page, int n_units) {
+    __shared__ float part[2][WAVES][64][4];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = lane & 15, q = lane >> 4;
+    const int s0 = wave * KSTEPS;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    const int k8_last = (K >> 3) - 1;
+    const int half = d >> 1, upt = d >> 5;   // units per head slot
+    uint4 xf[KSTEPS];
+    int k8c[KSTEPS];
+    {
+        const uint4* xp = reinterpret_cast<const uint4*>(X + (size_t)(r < M ? r : 0) * lda);
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u) {
+            const int k8 = (s0 + u) * 4 + q;
+            k8c[u] = k8 < k8_last ? k8 : k8_last;
+            const uint4 v = xp[k8c[u]];
+            xf[u] = (k8 <= k8_last && r < M) ? v : zero;   // zero fragments make the clamped W loads harmless
+        }
+    }
+    // first W row of tile `half_idx` (0, 1) of unit u
+    auto tile_row = [&](int u, int half_idx) -> int { return (u / upt) * d + (u % upt) * 16 + half_idx * half; };
+    uint4 a[KSTEPS];
+    int unit = blockIdx.x;
+    if (unit < n_units) {
+        const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)(tile_row(unit, 0) + r) * ldw);
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
+    }
+    // the epilogue thread's output: row m, column nl of a tile
+    const int et = threadIdx.x < 256 ? threadIdx.x : 0;
+    const int e = et & 3, l = et >> 2;
+    const int m = l & 15, nl = (l >> 4) * 4 + e;
+    const bool writer = threadIdx.x < 256 && m < M;
+    const int p_m = writer ? pos[m] : 0;
+    const int slot = (writer && slots != nullptr) ? slots[m] : -1;
+    int buf = 0;
+    for (; unit < n_units; unit += gridDim.x) {
+        const int hs = unit / upt, j = unit % upt;
+        const int i0 = j * 16 + nl;   // this thread's dim within the first half of the head
+        float cs = 1.f, sn = 0.f;
+        if (writer && hs < nh + nkv) {   // on their way while the products run
+            cs = cosT[(size_t)p_m * half + i0];
+            sn = sinT[(size_t)p_m * half + i0];
+        }
+        float val[2];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < KSTEPS; ++u) acc = qr_mfma(a[u], xf[u], acc);
+            // the next tile's rows are on their way while this one is reduced
+            const int nu = hf == 0 ? unit : unit + gridDim.x;
+            __builtin_amdgcn_sched_barrier(0);
+            if (nu < n_units) {
+                const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)(tile_row(nu, hf == 0 ? 1 : 0) + r) * ldw);
+#pragma unroll
+                for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            *reinterpret_cast<f32x4*>(&part[buf][wave][lane][0]) = acc;
+            __syncthreads();
+            float v = 0.f;
+            if (threadIdx.x < 256) {
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) v += part[buf][w][l][e];
+                if (bias != nullptr) v += to_f32(bias[tile_row(unit, hf) + nl]);
+            }
+            val[hf] = qr_round(v);
+            buf ^= 1;  // the other buffer is free: its readers passed the barrier above one tile ago
+        }
+        if (!writer) continue;
+        if (hs < nh + nkv) {
+            const float ra = val[0] * cs - val[1] * sn;
+            const float rb = val[1] * cs + val[0] * sn;
+            if (hs < nh) {
+                bf16* dst = Q + (size_t)m * ldq + (size_t)hs * d + i0;
+                dst[0] = from_f32<bf16>(ra);
+                dst[half] = from_f32<bf16>(rb);
+            } else if (slot >= 0) {
+                bf16* dst = kc + (((size_t)(slot / page) * nkv + (hs - nh)) * page + (slot % page)) * d + i0;
+                dst[0] = from_f32<bf16>(ra);
+                dst[half] = from_f32<bf16>(rb);
+            }
+        } else if (slot >= 0) {
+            // values are cached transposed, [pages, nkv, d, page]
+            bf16* dst = vc + ((size_t)(slot / page) * nkv + (hs - nh - nkv)) * d * page + (slot % page);
+            dst[(size_t)i0 * page] = from_f32<bf16>(val[0]);
+            dst[(size_t)(i0 + half) * page] = from_f32<bf16>(val[1]);
+        }
+    }
+}
+
+static int qr_num_cus() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
+// Q [M, ldq] receives the rotated query heads; k (rotated) and v go to the cache slots (slots may be
+// null: nothing is cached).  W [(nh + 2 nkv) d, ldw] holds the q, k, v rows in this order.
+extern "C" int ilm_gemm_qkv_rope(void* Q, int ldq, const void* X, int lda, const void* W, int ldw, const void* bias,
+                                 int M, int K, const void* pos, const void* cosT, const void* sinT, void* kc, void* vc,
+                                 const void* slots, int nh, int nkv, int d, int page, hipStream_t stream) {
+    ILM_REQUIRE(M > 0 && M <= 16 && K > 0 && nh > 0 && nkv >= 0, "gemm_qkv_rope: needs 1 <= M <= 16, got M=%d K=%d", M, K);
+    ILM_REQUIRE(d > 0 && d % 32 == 0, "gemm_qkv_rope: head size %d is not a multiple of 32", d);
+    ILM_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldq >= nh * d,
+                "gemm_qkv_rope: K=%d lda=%d ldw=%d ldq=%d", K, lda, ldw, ldq);
+    ILM_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_qkv_rope: operands must be 16-byte aligned");
+    ILM_REQUIRE(slots == nullptr || (page > 0 && kc != nullptr && vc != nullptr), "gemm_qkv_rope: cache missing");
+    const int ksteps = (K + 31) / 32;
+    ILM_REQUIRE(ksteps <= 16 * 16, "gemm_qkv_rope: K=%d is beyond 8192", K);
+    const int n_units = (nh + 2 * nkv) * (d / 32);
+#define QR_CASE(WV, KS)                                                                                        \
+    {                                                                                                          \
+        const int cap = qr_num_cus() * (WV == 16 ? 1 : 2);                                                     \
+        const int grid = n_units < cap ? n_units : cap;                                                        \
+        gemm_qkv_rope_kernel<WV, KS><<<grid, WV * 64, 0, stream>>>(                                            \
+            (bf16*)Q, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, K, lda, ldw, ldq, (const int*)pos, \
+            (const float*)cosT, (const float*)sinT, (bf16*)kc, (bf16*)vc, (const int*)slots, nh, nkv, d, page, \
+            n_units);                                                                                          \
+    }
+    if (ksteps <= 8 * 4) QR_CASE(8, 4)
+    else if (ksteps <= 8 * 8) QR_CASE(8, 8)
+    else if (ksteps <= 16 * 8) QR_CASE(16, 8)
+    else QR_CASE(16, 16)
+#undef QR_CASE
+    ILM_LAUNCH_CHECK("gemm_qkv_rope");
+    return 0;
+}

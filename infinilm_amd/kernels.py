@@ -196,6 +196,43 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, 
          _ptr(v_cache), _ptr(slots), T, nh, nkv, d, rd, qkv.stride(0), page, _dt(qkv), _stream())
 
 
+USE_QKV_ROPE = os.environ.get("INFINILM_AMD_QKV_ROPE", "1") == "1"
+
+
+def qkv_rope_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
+                  cos: torch.Tensor, sin: torch.Tensor, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                  slots: Optional[torch.Tensor], nh: int, nkv: int, d: int, rd: int) -> Optional[torch.Tensor]:
+    """The fused projection x w^T (+ bias) of a few rows, q and k rotated and k, v written to the cache
+    in the product's epilogue.  Returns the rotated q [T, nh*d], or None where the fused kernel does
+    not apply (more than 16 rows, float32, a partly rotated or odd-sized head): the caller then
+    runs the projection and `rope_kvwrite` one after the other."""
+    M, K = x.shape
+    if not (USE_QKV_ROPE and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and M <= 16 and rd == d and d % 32 == 0
+            and K % 8 == 0 and K <= 8192 and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
+            and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        return None
+    _dev(x, w, bias, positions, cos, sin, k_cache, v_cache, slots)
+    _i32(positions, "positions")
+    if w.shape != ((nh + 2 * nkv) * d, K) or positions.numel() != M:
+        raise KernelError(f"fused projection {tuple(w.shape)} does not fit {nh}+2*{nkv} heads of {d} over {K}")
+    if bias is not None and (bias.shape != (w.shape[0],) or bias.dtype != BF16 or not bias.is_contiguous()):
+        raise KernelError("bias does not fit the fused projection")
+    if cos.dtype != F32 or sin.dtype != F32 or cos.shape != sin.shape or cos.shape[1] != d // 2 \
+            or not cos.is_contiguous() or not sin.is_contiguous():
+        raise KernelError(f"rotation tables must be float32 [positions, {d // 2}], got {tuple(cos.shape)}")
+    page = 0
+    if slots is not None:
+        _i32(slots, "slots")
+        if k_cache is None or v_cache is None or k_cache.dtype != BF16 or v_cache.dtype != BF16:
+            raise KernelError("cache tensors missing or of another dtype than the activations")
+        page = _check_cache(k_cache, v_cache, nkv, d)
+    q = torch.empty((M, nh * d), dtype=BF16, device=x.device)
+    _run("ilm_gemm_qkv_rope", q.data_ptr(), q.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), _ptr(bias),
+         M, K, positions.data_ptr(), cos.data_ptr(), sin.data_ptr(), _ptr(k_cache) if slots is not None else None,
+         _ptr(v_cache) if slots is not None else None, _ptr(slots), nh, nkv, d, page, _stream())
+    return q
+
+
 def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     """silu(gate) * up from rows [gate | up]."""
     _dev(gate_up)

@@ -47,11 +47,18 @@ class GQAttention(Mixer):
     def forward(self, x: torch.Tensor, batch, cache_view) -> torch.Tensor:
         if batch.max_position >= self.position.max_positions:
             raise ValueError(f"position {batch.max_position} is beyond the position table ({self.position.max_positions})")
-        qkv = self.qkv.forward(x)
-        kernels.rope_kvwrite(qkv, batch.positions, self.position.cos, self.position.sin, cache_view.k, cache_view.v,
-                             cache_view.slots, self.nh, self.nkv, self.d, self.position.rotary_dim)
-        if batch.taps is not None:
-            batch.taps.setdefault("qkv_rotated", []).append(qkv.clone())
+        # few rows (decoded tokens): projection, rotation and cache write are one kernel
+        qkv = None
+        if batch.taps is None and isinstance(self.position.cos, torch.Tensor):
+            qkv = kernels.qkv_rope_gemm(x, self.qkv.weight, self.qkv.bias, batch.positions, self.position.cos,
+                                        self.position.sin, cache_view.k, cache_view.v, cache_view.slots, self.nh,
+                                        self.nkv, self.d, self.position.rotary_dim)
+        if qkv is None:
+            qkv = self.qkv.forward(x)
+            kernels.rope_kvwrite(qkv, batch.positions, self.position.cos, self.position.sin, cache_view.k, cache_view.v,
+                                 cache_view.slots, self.nh, self.nkv, self.d, self.position.rotary_dim)
+            if batch.taps is not None:
+                batch.taps.setdefault("qkv_rotated", []).append(qkv.clone())
         o = kernels.paged_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,
                                     batch.positions, self.nh, self.nkv, self.d, self.scale, self.window,
                                     batch.max_total_len, batch.att_tiles, batch.att_single_rows)

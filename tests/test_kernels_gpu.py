@@ -103,6 +103,56 @@ def test_rope_and_cache_write(K, dtype, nh, nkv, d, rd, page):
     assert not kc.cpu().permute(0, 2, 1, 3).reshape(n_pages * page, -1)[mask].any()  # nothing else was touched
 
 
+@pytest.mark.parametrize("M,nh,nkv,d,Kd,page,bias", [(5, 4, 2, 32, 96, 8, False), (16, 32, 2, 128, 4096, 64, False),
+                                                     (1, 3, 3, 64, 200, 16, True), (8, 16, 2, 64, 1024, 16, False),
+                                                     (3, 2, 1, 96, 8192, 4, True)])
+def test_projection_with_rotation_and_cache_write_in_one_kernel(K, M, nh, nkv, d, Kd, page, bias):
+    """The decode-side fused kernel against the plain product + rotation, and against the
+    product kernel followed by the rotation kernel."""
+    max_pos = 300
+    N = (nh + 2 * nkv) * d
+    x, w = _rand((M, Kd), 21, torch.bfloat16), _rand((N, Kd), 22, torch.bfloat16, scale=Kd ** -0.5)
+    b = _rand((N,), 23, torch.bfloat16) if bias else None
+    g = torch.Generator().manual_seed(24)
+    pos = torch.randint(0, max_pos, (M,), generator=g, dtype=torch.int32)
+    pos[0] = max_pos - 1
+    cfg = {"hidden_size": d, "num_attention_heads": 1, "max_position_embeddings": max_pos, "rope_theta": 5000.0}
+    cos, sin = P.plain_rope_tables(cfg)
+    n_pages = M + 2
+    slots = (torch.randperm(n_pages, generator=g)[:M] * page + torch.randint(0, page, (M,), generator=g)).to(torch.int32)
+    if M > 2:
+        slots[2] = -1   # a token that is not cached
+    dev = lambda t: None if t is None else t.to(DEV)
+    caches = []
+    for fused in (True, False):
+        kc = torch.zeros((n_pages, nkv, page, d), dtype=torch.bfloat16, device=DEV)
+        vc = torch.zeros((n_pages, nkv, d, page), dtype=torch.bfloat16, device=DEV)
+        if fused:
+            q = K.qkv_rope_gemm(dev(x), dev(w), dev(b), dev(pos), dev(cos.float()), dev(sin.float()), kc, vc, dev(slots),
+                                nh, nkv, d, d)
+            assert q is not None
+        else:
+            qkv = K.gemm(dev(x), dev(w), dev(b))
+            K.rope_kvwrite(qkv, dev(pos), dev(cos.float()), dev(sin.float()), kc, vc, dev(slots), nh, nkv, d, d)
+            q = qkv[:, :nh * d]
+        caches.append((q.cpu().float(), kc.cpu().float(), vc.cpu().float()))
+    y = P.plain_linear(x.to(F64), w.to(F64), None if b is None else b.to(F64)).view(M, nh + 2 * nkv, d)
+    want_q = P.plain_apply_rope(y[:, :nh], pos, cos, sin, d).reshape(M, nh * d)
+    want_k = P.plain_apply_rope(y[:, nh:nh + nkv], pos, cos, sin, d)
+    q, kc, vc = caches[0]
+    _close(q, want_q, 1e-2)
+    for t in range(M):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        _close(kc[s // page, :, s % page, :], want_k[t], 1e-2)
+        _close(vc[s // page, :, :, s % page], y[t, nh + nkv:], 1e-2)
+    # the two paths round the projection to bfloat16 at the same place: they agree to an ulp of the result
+    for a, b_ in zip(caches[0], caches[1]):
+        assert (a - b_).abs().max() <= 2 ** -7 * max(a.abs().max(), 1e-6)
+        assert ((a != 0) == (b_ != 0)).all()   # and write the same places, nothing else
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu_and_gather(K, dtype):
     gu = _rand((7, 2 * 200), 6, dtype, 2.0)
