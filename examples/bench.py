@@ -66,7 +66,9 @@ def run_case(llm: LLM, case: dict, seed: int, sp_kwargs: dict) -> dict:
         if t_first_all is None and len(first) == len(reqs):
             t_first_all = now
             steps_at_first = steps
+            mid = eng.stats()
     t1 = time.perf_counter()
+    after = eng.stats()
     failed = [r.error for r in reqs if r.error]
     if failed:
         return dict(case, error=failed[0])
@@ -79,7 +81,11 @@ def run_case(llm: LLM, case: dict, seed: int, sp_kwargs: dict) -> dict:
                 prefill_tok_s=round(b * n_in / prefill_s, 1),
                 decode_tok_s=round(decode_tokens / decode_s, 1) if decode_tokens > 0 and decode_s > 0 else None,
                 decode_ms_per_step=round(1e3 * decode_s / max(steps - steps_at_first, 1), 3),
-                total_ms=round(1e3 * (t1 - t0), 2))
+                total_ms=round(1e3 * (t1 - t0), 2),
+                # host milliseconds of a decode step: scheduling, building and launching the step,
+                # bookkeeping (the wait for the device is inside the sampler's copy of the tokens: not counted)
+                decode_host_ms_per_step=round(1e3 * sum(after[k] - mid[k] for k in ("schedule_s", "step_s", "update_s"))
+                                              / max(steps - steps_at_first, 1), 3))
 
 
 def main(argv=None) -> int:

@@ -65,7 +65,7 @@ class LLMEngine:
             return []
         entries = []
         for e in out.entries:
-            toks = e.request.all_token_ids()[e.start:e.start + e.num_tokens]
+            toks = e.request.token_slice(e.start, e.num_tokens)
             entries.append(StepEntry(e.request.request_id, toks, [e.num_tokens - 1] if e.samples else []))
         logits = self.runner.step(entries)
         t2 = time.perf_counter()

@@ -67,6 +67,15 @@ class InferenceRequest:
     def all_token_ids(self) -> List[int]:
         return self.prompt_token_ids + self.output_token_ids
 
+    def token_slice(self, start: int, n: int) -> List[int]:
+        """all_token_ids()[start:start + n] without joining the two lists."""
+        lp = len(self.prompt_token_ids)
+        if start >= lp:
+            return self.output_token_ids[start - lp:start - lp + n]
+        if start + n <= lp:
+            return self.prompt_token_ids[start:start + n]
+        return self.prompt_token_ids[start:] + self.output_token_ids[:start + n - lp]
+
     def num_known_tokens(self) -> int:
         return len(self.prompt_token_ids) + len(self.output_token_ids)
 

@@ -66,7 +66,7 @@ class Scheduler:
         self.finished: List[InferenceRequest] = []
         self._admissions = 0
         self.num_preemptions = 0
-        self.log: List[Dict] = []  # composition of each step
+        self.log: Deque[Dict] = deque(maxlen=4096)  # composition of the latest steps
 
     # ---- adding ---------------------------------------------------------------------------------
     def _pages_for(self, n_tokens: int) -> int:
@@ -139,16 +139,20 @@ class Scheduler:
         promised = [0] * len(self.cache.groups)
         budget = self.max_num_batched_tokens
 
+        planned_ids = set()
+        gone = set()      # requests taken out of `running` during this call
+
         def plan(req: InferenceRequest, n: int) -> None:
             nonlocal budget
             start = req.num_computed_tokens
             self._promise(req, n, promised)
             out.entries.append(ScheduledEntry(req, start, n, start + n == req.num_known_tokens()))
+            planned_ids.add(id(req))
             budget -= n
 
         # 1. decode tokens of running requests, oldest first; make room by preempting the newest
         for req in sorted(self.running, key=lambda r: r.admission_index):
-            if req not in self.running:       # preempted while serving an older one
+            if id(req) in gone:               # preempted while serving an older one
                 continue
             if req.num_known_tokens() - req.num_computed_tokens != 1 or req.get_num_generated_tokens() == 0:
                 continue
@@ -160,20 +164,23 @@ class Scheduler:
                     # alone with the whole pool and still short of a page: it can never finish
                     self.cache.release(req.request_id)
                     self.running.remove(req)
+                    gone.add(id(req))
                     self._fail(req, "no_capacity: the request cannot make progress with the whole pool to itself")
                     break
                 planned = [e for e in out.entries if e.request is victim]
                 if planned:                   # never happens for decodes planned oldest-first, kept for safety
                     out.entries.remove(planned[0])
+                    planned_ids.discard(id(victim))
                 self._preempt(victim, out)
+                gone.add(id(victim))
                 if victim is req:
                     break
-            if req in self.running:
+            if id(req) not in gone:
                 plan(req, 1)
         # 2. portions of prompts already begun (and recomputations after a preemption)
         for req in sorted(self.running, key=lambda r: r.admission_index):
             left = req.num_known_tokens() - req.num_computed_tokens
-            if any(e.request is req for e in out.entries) or left <= 0 or budget <= 0:
+            if id(req) in planned_ids or left <= 0 or budget <= 0:
                 continue
             n = min(left, self.chunk_size, budget)
             while n > 0 and not self._fits(req, n, promised):

@@ -171,10 +171,15 @@ class StepRunner:
         seg("token_ids")[:] = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=T)
         pos = seg("positions")
         sot = seg("seg_of_token")
-        for i in range(R):
-            a, b = offsets[i], offsets[i + 1]
-            pos[a:b] = np.arange(start[i], start[i] + lens[i])
-            sot[a:b] = i
+        all_single = T == R
+        if all_single:   # decoded tokens only: no per-entry array work
+            pos[:] = start
+            sot[:] = np.arange(R)
+        else:
+            for i in range(R):
+                a, b = offsets[i], offsets[i + 1]
+                pos[a:b] = np.arange(start[i], start[i] + lens[i])
+                sot[a:b] = i
         seg("seg_offsets")[:] = offsets
         seg("start_pos")[:] = start
         seg("total_lens")[:] = start + lens
@@ -193,6 +198,18 @@ class StepRunner:
             sl = seg(f"slots{g}")
             bt = seg(f"bt{g}").reshape(R, max_blocks[g])
             bt[:] = -1
+            if all_single:
+                slot_list = []
+                for i, e in enumerate(entries):
+                    table = cache.table(e.req_id, g)
+                    bt[i, :len(table)] = table
+                    p = int(start[i])
+                    page = table[p // ps]
+                    if page < 0:
+                        raise RuntimeError(f"request {e.req_id!r}: a new token falls on a page already given back")
+                    slot_list.append(page * ps + p % ps)
+                sl[:] = slot_list
+                continue
             for i, e in enumerate(entries):
                 table = np.asarray(cache.table(e.req_id, g), dtype=np.int64)
                 bt[i, :len(table)] = table

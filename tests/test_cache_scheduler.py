@@ -305,3 +305,12 @@ def test_every_admitted_request_finishes_under_random_load(seed):
     assert all(r.get_num_generated_tokens() == r.sampling_params.max_tokens for r in ok)
     assert all("no_capacity" in r.error for r in reqs if r.status == RequestStatus.FAILED)
     assert c.free_pages() == 14 and not c.requests
+
+
+def test_token_slice_equals_a_slice_of_all_tokens():
+    r = _req("a", 4, max_tokens=9)
+    r.output_token_ids = [5, 6, 7]
+    joined = r.all_token_ids()
+    for s in range(7):
+        for n in range(1, 8 - s):
+            assert r.token_slice(s, n) == joined[s:s + n]
