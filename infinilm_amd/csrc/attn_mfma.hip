@@ -294,12 +294,7 @@ attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, cons
 #define ATT_BT_LDS 2048  // block-table entries kept in LDS
 #define ATT_LAZY 8.0f    // the exponent's reference point follows the maximum in steps of at least this
 
-// maximum of three without the quieting of NaN that fmaxf brings (scores are finite)
-__device__ __forceinline__ float max3(float a, float b, float c) {
-    float d;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
-    return d;
-}
+__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 
 template <int D16, bool PAGE64>
 __global__ void __launch_bounds__(256, 2)
@@ -445,10 +440,168 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     const int kb0 = lo_first & ~(ATT_TK - 1);
     __syncthreads();   // bt_s is filled
     ATT_FETCH(kb0)
-    for (int kb = kb0; kb <= p_last; kb += ATT_TK) {
+    // every tile begins with the exchange of the staged registers for the tile in LDS
+    auto tile_begin = [&]() {
         __syncthreads();   // the previous tile has been consumed
         ATT_STASH()
         __syncthreads();
+    };
+    // A tile that both tokens of the wave see whole (every tile but those on the diagonal and at a
+    // window's edge) takes a path without masks, written so that matrix and vector instructions
+    // alternate: a wave issues in order, so the vector work of one sub-tile has to stand between
+    // the matrix instructions of another to run beside them.
+    auto fast_tile = [&](int kb) {
+        uint4 kf0[2][KS], kf1[2][KS];
+        f32x4 s0[ATT_NT][2], s1[ATT_NT][2];
+#pragma unroll
+        for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) kf0[tau][ks] = *reinterpret_cast<const uint4*>(&Ks[tau * 16 + r][ks * 32 + qg * 8]);
+#pragma unroll
+        for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+            for (int j = 0; j < ATT_NT; ++j) {
+                s0[j][tau] = f32x4{0.f, 0.f, 0.f, 0.f};
+                s1[j][tau] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+                for (int j = 0; j < ATT_NT; ++j) s0[j][tau] = mfma16(kf0[tau][ks], qf[j][ks], s0[j][tau]);
+        __builtin_amdgcn_sched_barrier(0);   // the next fragments take the registers of these
+#pragma unroll
+        for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) kf1[tau][ks] = *reinterpret_cast<const uint4*>(&Ks[32 + tau * 16 + r][ks * 32 + qg * 8]);
+        // the reference point of the exponent follows the maximum lazily (see below); rare
+#define ATT_FOLLOW(S_, PRE_)                                                                               \
+        {                                                                                                  \
+            /* scores become exponents relative to the reference point, in place */                       \
+            float lm[ATT_NT];                                                                              \
+            bool over = false;                                                                             \
+            _Pragma("unroll") for (int j = 0; j < ATT_NT; ++j) {                                           \
+                const bool unset = mc[j] < 0.5f * NEG_BIG;   /* no key seen yet: exponents relative to 0 */ \
+                const float nm = unset ? 0.f : -mc[j];                                                     \
+                _Pragma("unroll") for (int tau = 0; tau < 2; ++tau)                                        \
+                    _Pragma("unroll") for (int e = 0; e < 4; ++e) S_[j][tau][e] = fmaf(S_[j][tau][e], scale_log2e, nm); \
+                lm[j] = max3(max3(S_[j][0][0], S_[j][0][1], S_[j][0][2]), max3(S_[j][0][3], S_[j][1][0], S_[j][1][1]), \
+                             fmaxf(S_[j][1][2], S_[j][1][3]));                                             \
+                over = over || unset || lm[j] > ATT_LAZY;                                                  \
+            }                                                                                              \
+            if (__builtin_amdgcn_ballot_w64(over) != 0ull) {                                               \
+                PRE_                                                                                       \
+                _Pragma("unroll") for (int j = 0; j < ATT_NT; ++j) {                                       \
+                    float mx = lm[j];                                                                      \
+                    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));                                                \
+                    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));                                                \
+                    const bool unset = mc[j] < 0.5f * NEG_BIG;                                             \
+                    const bool up = unset || mx > ATT_LAZY;   /* the same in the four lanes of a column */ \
+                    const float shift = up ? mx : 0.f;                                                     \
+                    const float corr = unset ? 1.0f : __builtin_amdgcn_exp2f(-shift);   /* unset: sums are 0 */ \
+                    mc[j] = unset ? mx : mc[j] + shift;                                                    \
+                    _Pragma("unroll") for (int tau = 0; tau < 2; ++tau)                                    \
+                        _Pragma("unroll") for (int e = 0; e < 4; ++e) S_[j][tau][e] -= shift;              \
+                    _Pragma("unroll") for (int e = 0; e < 4; ++e) lacc[j][e] *= corr;                      \
+                    _Pragma("unroll") for (int db = 0; db < D16; ++db)                                     \
+                        _Pragma("unroll") for (int e = 0; e < 4; ++e) acc[j][db][e] *= corr;               \
+                }                                                                                          \
+            }                                                                                              \
+        }
+        // one quarter of a sub-tile's p: token J_, key tile TAU_ -> two words of its fragment
+#define ATT_PQ(S_, J_, TAU_, LO_, HI_)                                                                     \
+        {                                                                                                  \
+            const float p0 = __builtin_amdgcn_exp2f(S_[J_][TAU_][0]);                                      \
+            const float p1 = __builtin_amdgcn_exp2f(S_[J_][TAU_][1]);                                      \
+            const float p2 = __builtin_amdgcn_exp2f(S_[J_][TAU_][2]);                                      \
+            const float p3 = __builtin_amdgcn_exp2f(S_[J_][TAU_][3]);                                      \
+            LO_ = pack_bf16x2(p0, p1);                                                                     \
+            HI_ = pack_bf16x2(p2, p3);                                                                     \
+        }
+        ATT_FOLLOW(s0, )
+        // scores of the second sub-tile on the matrix cores, p of the first on the vector units
+        uint4 pf0[ATT_NT], pf1[ATT_NT];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+            for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+                for (int j = 0; j < ATT_NT; ++j) s1[j][tau] = mfma16(kf1[tau][ks], qf[j][ks], s1[j][tau]);
+            if (ks == 0) ATT_PQ(s0, 0, 0, pf0[0].x, pf0[0].y)
+            if (ks == 1 || KS == 1) ATT_PQ(s0, 0, 1, pf0[0].z, pf0[0].w)
+            if (ks == 2 || (KS <= 2 && ks == KS - 1)) ATT_PQ(s0, 1, 0, pf0[1].x, pf0[1].y)
+            if (ks == KS - 1) ATT_PQ(s0, 1, 1, pf0[1].z, pf0[1].w)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // the next tile leaves for the registers only now: until here they held score fragments
+        if (kb + ATT_TK <= p_last) { ATT_FETCH(kb + ATT_TK) }
+        // values of the first sub-tile; their products stand between the p of the second
+        // (should the reference point move now, the first sub-tile's products, made with the old one,
+        // are added first, and the interleaved block below adds zeros in their place)
+        ATT_FOLLOW(s1, {
+            _Pragma("unroll") for (int j = 0; j < ATT_NT; ++j) lacc[j] = mfma16(ones4, pf0[j], lacc[j]);
+            _Pragma("unroll") for (int db = 0; db < D16; ++db) {
+                const uint4 v = *reinterpret_cast<const uint4*>(&Vs[db * 16 + r][qg * 8]);
+                _Pragma("unroll") for (int j = 0; j < ATT_NT; ++j) acc[j][db] = mfma16(v, pf0[j], acc[j][db]);
+            }
+            _Pragma("unroll") for (int j = 0; j < ATT_NT; ++j) pf0[j] = zero4;
+        })
+        constexpr int DH = (D16 + 1) / 2;   // value fragments in two halves: fewer registers live
+        uint4 vf[DH];
+#pragma unroll
+        for (int db = 0; db < DH; ++db) vf[db] = *reinterpret_cast<const uint4*>(&Vs[db * 16 + r][qg * 8]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < ATT_NT; ++j) lacc[j] = mfma16(ones4, pf0[j], lacc[j]);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int i = 0; i < DH; ++i) {
+                const int db = h * DH + i;
+                if (db < D16) {
+#pragma unroll
+                    for (int j = 0; j < ATT_NT; ++j) acc[j][db] = mfma16(vf[i], pf0[j], acc[j][db]);
+                }
+                if (h == 0 && i == 0) ATT_PQ(s1, 0, 0, pf1[0].x, pf1[0].y)
+                if (h == 0 && i == DH - 1) ATT_PQ(s1, 0, 1, pf1[0].z, pf1[0].w)
+                if (h == 1 && i == 0) ATT_PQ(s1, 1, 0, pf1[1].x, pf1[1].y)
+                if (h == 1 && i == DH - 1) ATT_PQ(s1, 1, 1, pf1[1].z, pf1[1].w)
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // the next half: second half of this sub-tile, then the first of the other
+#pragma unroll
+            for (int i = 0; i < DH; ++i) {
+                const int db = (h == 0 ? DH : 0) + i;
+                if (db < D16) vf[i] = *reinterpret_cast<const uint4*>(&Vs[db * 16 + r][(h == 0 ? 0 : 32) + qg * 8]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < ATT_NT; ++j) lacc[j] = mfma16(ones4, pf1[j], lacc[j]);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int i = 0; i < DH; ++i) {
+                const int db = h * DH + i;
+                if (db < D16) {
+#pragma unroll
+                    for (int j = 0; j < ATT_NT; ++j) acc[j][db] = mfma16(vf[i], pf1[j], acc[j][db]);
+                }
+            }
+            if (h == 0) {
+#pragma unroll
+                for (int i = 0; i < DH; ++i) {
+                    const int db = DH + i;
+                    if (db < D16) vf[i] = *reinterpret_cast<const uint4*>(&Vs[db * 16 + r][32 + qg * 8]);
+                }
+            }
+        }
+#undef ATT_FOLLOW
+#undef ATT_PQ
+    };
+    // any tile: masks where a token does not see a key
+    auto general_tile = [&](int kb) {
         if (kb + ATT_TK <= p_last) { ATT_FETCH(kb + ATT_TK) }   // in flight while this tile is multiplied
         // The score products of both 32-key sub-tiles are issued first, so that the matrix cores
         // work on the second while the vector units do the softmax of the first.
@@ -555,6 +708,26 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
                 for (int j = 0; j < ATT_NT; ++j) acc[j][db] = mfma16(vf, pf[j], acc[j][db]);
             }
         }
+    };
+    // Tiles [kb_a, kb_b) are seen whole by every token of the workgroup: from the window's edge of the
+    // last token (the start without a window) to the tile before the first token's own.  Three loops
+    // rather than one with a branch: each keeps its own registers.
+    const int lo_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+    int kb_a = (lo_last + ATT_TK - 1) & ~(ATT_TK - 1);
+    int kb_b = ((p_first + 1) / ATT_TK) * ATT_TK;
+    if (D % 32 != 0 || kb_b < kb_a) kb_a = kb_b = kb0;
+    int kb = kb0;
+    for (; kb < kb_a && kb <= p_last; kb += ATT_TK) {
+        tile_begin();
+        general_tile(kb);
+    }
+    for (; kb < kb_b; kb += ATT_TK) {
+        tile_begin();
+        fast_tile(kb);
+    }
+    for (; kb <= p_last; kb += ATT_TK) {
+        tile_begin();
+        general_tile(kb);
     }
     if (!head_ok) return;
 #pragma unroll
