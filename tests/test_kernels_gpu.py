@@ -368,6 +368,18 @@ def test_argmax_and_sampling(K):
             assert dist[tok] > 0, f"token {tok} is outside the kept set (T={temp}, k={k}, p={p})"
             lo = float(cdf[tok] - dist[tok])
             assert lo - 1e-4 <= u <= float(cdf[tok]) + 1e-4, f"u={u} not in token {tok}'s interval"
+    # every row length takes its own kernel shape (row in registers of 1024 or 512 threads, or streamed)
+    for Vn in (16384, 20000, 40000, 73448, 90000, 122753):
+        big = _rand((1, Vn), 30 + Vn % 7, scale=2.5)
+        for temp, k, p in [(0.9, 0, 1.0), (1.1, 50, 0.9), (1.0, 0, 0.7), (0.6, 7, 1.0)]:
+            dist = P.plain_sample_distribution(big[0], temp, k, p)
+            cdf = torch.cumsum(dist, 0)
+            us = [i / 8.0 + 1 / 16.0 for i in range(8)]
+            got = run(temp, k, p, us, big.expand(8, Vn).contiguous())
+            for u, tok in zip(us, got):
+                assert dist[tok] > 0, f"V={Vn}: token {tok} is outside the kept set (T={temp}, k={k}, p={p})"
+                lo = float(cdf[tok] - dist[tok])
+                assert lo - 2e-4 <= u <= float(cdf[tok]) + 2e-4, f"V={Vn}: u={u} not in token {tok}'s interval"
     # frequencies over many draws follow the probabilities
     dist = P.plain_sample_distribution(small[0], 1.0, 8, 1.0)
     n = 4096
