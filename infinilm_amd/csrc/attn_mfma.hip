@@ -3,12 +3,15 @@
 // Same contract as attn_basic.hip.  Two kernels: single tokens (decoding) over key chunks, below,
 // and tiles of consecutive tokens of one request (portions of prompts), further down.
 //
-// Single tokens: `rows` (optional) lists the token rows to serve.  A workgroup of 4 waves serves one token and one group of up to
-// 16 query heads that share a KV head, over one chunk of ATT_CHUNK keys; each wave takes a quarter
-// of the chunk, the four partial results are merged through LDS.  Chunks are aligned to absolute
-// key index, so what is summed in which order depends on (request, position) alone.  With more
-// than one chunk the partial results (max, sum, unnormalised output) go to a workspace and a
-// second kernel merges them in chunk order.
+// Single tokens: `rows` (optional) lists the token rows to serve.  A workgroup of 4 waves serves one
+// token and one group of up to 16 query heads that share a KV head, over one chunk of `span` keys
+// (a multiple of ATT_STEP = 128, chosen by the caller so that the launch fills the chip: short
+// chunks for few tokens, long ones for many).  The chunk is walked in steps of 128 keys, 32 a wave,
+// the loads of the next step in flight while this one is multiplied; the four waves' partial
+// results are merged through LDS.  Chunks are aligned to absolute key index.  With more than one
+// chunk the partial results (max, sum, unnormalised output) go to a workspace and a second kernel
+// merges them in chunk order.  For a given chunk length the result depends on (request, position)
+// alone; another chunk length changes the order of summation, not more.
 //
 // Per 32 keys:  S^T[keys x heads] = K Q^T   (v_mfma_f32_16x16x32_bf16, K rows on the A side, read
 //                                            straight from the cache; d is the reduced dimension)
@@ -17,18 +20,15 @@
 //                                            consecutive keys of one dim are one 16-byte load)
 // The rows of the two S tiles are assigned to keys so that each lane ends up with the
 // probabilities of 8 consecutive keys: they feed the second product without leaving registers.
-// All loads of a wave's 64 keys (K and V) are issued before the first product; they are
-// unconditional 16-byte loads from clamped addresses, masked afterwards.
+// Loads are unconditional 16-byte loads from clamped addresses, masked afterwards.
 // Needs: head size a multiple of 16 up to 128, page size a multiple of 16.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-#define ATT_CHUNK 256
 #define ATT_WAVES 4
-#define ATT_WKEYS (ATT_CHUNK / ATT_WAVES)  // keys per wave
-#define ATT_ITERS (ATT_WKEYS / 32)
+#define ATT_STEP (ATT_WAVES * 32)  // keys a workgroup takes in one step; chunks are multiples of it
 #define NEG_BIG (-1.0e30f)
 
 typedef __attribute__((ext_vector_type(2))) float f32x2;
@@ -45,12 +45,12 @@ __device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
 }
 
 template <int D16>
-__global__ void __launch_bounds__(ATT_WAVES * 64)
+__global__ void __launch_bounds__(ATT_WAVES * 64, 2)
 attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
                  const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                  const int* __restrict__ block_tables, const int* __restrict__ seg,
                  const int* __restrict__ pos, const int* __restrict__ rows, int nh, int nkv, int page,
-                 int max_blocks, int q_stride, int out_stride, float scale_log2e, int window, int nsplit) {
+                 int max_blocks, int q_stride, int out_stride, float scale_log2e, int window, int nsplit, int span) {
     constexpr int D = D16 * 16;
     constexpr int KS = (D + 31) / 32;
     __shared__ float sm_acc[ATT_WAVES][D16][64][4];
@@ -60,30 +60,19 @@ attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __re
     const int HG = (G + 15) / 16;
     const int kvh = blockIdx.y / HG, hg = blockIdx.y % HG;
     const int split = blockIdx.z;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qg = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, r = lane & 15, qg = lane >> 4;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int hcol = hg * 16 + r;
     const bool head_ok = hcol < G;
     const int head = kvh * G + (head_ok ? hcol : G - 1);
 
-    // the chunk's valid keys [c_begin, c_end); empty: nothing to do for the whole workgroup
-    int c_begin = split * ATT_CHUNK, c_end = c_begin + ATT_CHUNK;
+    // the chunk's valid keys [c_begin, c_end); empty: nothing to do for the whole workgroup (the
+    // merge reads only the chunks between the first and the last key the token sees)
+    int c_begin = split * span, c_end = c_begin + span;
     if (c_begin < lo) c_begin = lo;
     if (c_end > p + 1) c_end = p + 1;
-    if (c_begin >= c_end) {
-        if (nsplit > 1 && head_ok && qg == 0 && wave == 0) {
-            float* ml = ws_ml + (((size_t)t * nh + head) * nsplit + split) * 2;
-            ml[0] = NEG_BIG;
-            ml[1] = 0.f;
-        }
-        return;
-    }
-    // this wave's keys [k_begin, k_end) within the chunk (may be empty)
-    const int w_base = split * ATT_CHUNK + wave * ATT_WKEYS;
-    const int k_begin = w_base > c_begin ? w_base : c_begin;
-    const int k_end = (w_base + ATT_WKEYS < c_end) ? w_base + ATT_WKEYS : c_end;
-    const bool wave_has_keys = k_begin < k_end;
+    if (c_begin >= c_end) return;
 
     const int* bt = block_tables + (size_t)seg[t] * max_blocks;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
@@ -92,9 +81,9 @@ attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __re
     for (int db = 0; db < D16; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m = NEG_BIG, lsum = 0.f;
 
-    if (wave_has_keys) {
-        // Q fragments: lane (r, qg) holds dims ks*32 + qg*8 .. +8 of head column r
-        uint4 qf[KS];
+    // Q fragments: lane (r, qg) holds dims ks*32 + qg*8 .. +8 of head column r
+    uint4 qf[KS];
+    {
         const bf16* qrow = q + (size_t)t * q_stride + (size_t)head * D;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
@@ -102,93 +91,101 @@ attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __re
             const uint4 v = *reinterpret_cast<const uint4*>(qrow + (dofs < D ? dofs : 0));
             qf[ks] = dofs < D ? v : zero4;
         }
-        // ---- every load of this wave's keys, issued at once
-        uint4 kf[ATT_ITERS][2][KS];
-        uint4 vf[ATT_ITERS][D16];
-#pragma unroll
-        for (int it = 0; it < ATT_ITERS; ++it) {
-            const int kb = w_base + it * 32;
-            // row i of S tile tau is key kb + (i/4)*8 + tau*4 + i%4; clamped onto pages that exist
-#pragma unroll
-            for (int tau = 0; tau < 2; ++tau) {
-                int key = kb + (r >> 2) * 8 + tau * 4 + (r & 3);
-                key = key < k_begin ? k_begin : (key >= k_end ? k_end - 1 : key);
-                const int pg = bt[key / page];
-                const bf16* krow = kc + (((size_t)pg * nkv + kvh) * page + (key % page)) * D;
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const int dofs = ks * 32 + qg * 8;
-                    kf[it][tau][ks] = *reinterpret_cast<const uint4*>(krow + (dofs < D ? dofs : 0));
-                }
-            }
-            // this lane's 8 keys of the second product are kb + qg*8 .. +8 (one page); a group with no
-            // valid key is read from the wave's first valid group instead and masked below
-            int key0 = kb + qg * 8;
-            if (key0 >= k_end || key0 + 8 <= k_begin) key0 = k_begin & ~7;
-            const int pg = bt[key0 / page];
-            const bf16* vbase = vc + ((size_t)pg * nkv + kvh) * D * page + (key0 % page);
-#pragma unroll
-            for (int db = 0; db < D16; ++db)
-                vf[it][db] = *reinterpret_cast<const uint4*>(vbase + (size_t)(db * 16 + r) * page);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int it = 0; it < ATT_ITERS; ++it) {
-            const int kb = w_base + it * 32;
-            if (kb >= k_end || kb + 32 <= k_begin) continue;  // wave-uniform
-            f32x4 s[2];
-#pragma unroll
-            for (int tau = 0; tau < 2; ++tau) {
-                s[tau] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const int dofs = ks * 32 + qg * 8;
-                    s[tau] = mfma16(dofs < D ? kf[it][tau][ks] : zero4, qf[ks], s[tau]);
-                }
-            }
-            // lane (r, qg) holds, for head column r, keys kb + qg*8 + tau*4 + e
-            float sv[8];
-            float mx = NEG_BIG;
-#pragma unroll
-            for (int tau = 0; tau < 2; ++tau)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int key = kb + qg * 8 + tau * 4 + e;
-                    const bool ok = key >= k_begin && key < k_end;
-                    const float v = ok ? s[tau][e] * scale_log2e : NEG_BIG;
-                    sv[tau * 4 + e] = v;
-                    mx = fmaxf(mx, v);
-                }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m, mx);
-            const float corr = __builtin_amdgcn_exp2f(m - m_new);
-            float pe[8];
-            float rs = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                pe[j] = (sv[j] > 0.5f * NEG_BIG) ? __builtin_amdgcn_exp2f(sv[j] - m_new) : 0.f;
-                rs += pe[j];
-            }
-            rs += __shfl_xor(rs, 16, 64);
-            rs += __shfl_xor(rs, 32, 64);
-            lsum = lsum * corr + rs;
-            m = m_new;
-            uint4 pf;
-            pf.x = pack_bf16x2(pe[0], pe[1]);
-            pf.y = pack_bf16x2(pe[2], pe[3]);
-            pf.z = pack_bf16x2(pe[4], pe[5]);
-            pf.w = pack_bf16x2(pe[6], pe[7]);
-            const int key0 = kb + qg * 8;
-            const bool vok = key0 < k_end && key0 + 8 > k_begin;  // else the loaded values are another group's
-#pragma unroll
-            for (int db = 0; db < D16; ++db) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc[db][e] *= corr;
-                acc[db] = mfma16(vok ? vf[it][db] : zero4, pf, acc[db]);
-            }
-        }
     }
+    // The chunk is walked in steps of ATT_STEP keys, 32 a wave; the loads of a step (K and V of the
+    // wave's 32 keys) are issued one step ahead into a second set of registers.  They are
+    // unconditional 16-byte loads from clamped addresses, masked afterwards.
+    const int first_step = (c_begin - split * span) / ATT_STEP, last_step = (c_end - 1 - split * span) / ATT_STEP;
+#define ATT_LOAD(KF_, VF_, STEP_)                                                                          \
+    {                                                                                                      \
+        const int kb_ = split * span + (STEP_) * ATT_STEP + wave * 32;                                     \
+        const int kbeg_ = kb_ > c_begin ? kb_ : c_begin, kend_ = kb_ + 32 < c_end ? kb_ + 32 : c_end;     \
+        if (kbeg_ < kend_) {   /* wave-uniform */                                                          \
+            _Pragma("unroll") for (int tau = 0; tau < 2; ++tau) {                                          \
+                /* row i of S tile tau is key kb + (i/4)*8 + tau*4 + i%4; clamped onto pages that exist */ \
+                int key = kb_ + (r >> 2) * 8 + tau * 4 + (r & 3);                                          \
+                key = key < kbeg_ ? kbeg_ : (key >= kend_ ? kend_ - 1 : key);                              \
+                const int pg = bt[key / page];                                                             \
+                const bf16* krow = kc + (((size_t)pg * nkv + kvh) * page + (key % page)) * D;              \
+                _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
+                    const int dofs = ks * 32 + qg * 8;                                                     \
+                    KF_[tau][ks] = *reinterpret_cast<const uint4*>(krow + (dofs < D ? dofs : 0));          \
+                }                                                                                          \
+            }                                                                                              \
+            /* this lane's 8 keys of the second product are kb + qg*8 .. +8 (one page); a group with no  \
+               valid key is read from the wave's first valid group instead and masked below */            \
+            int key0 = kb_ + qg * 8;                                                                       \
+            if (key0 >= kend_ || key0 + 8 <= kbeg_) key0 = kbeg_ & ~7;                                     \
+            const int pg = bt[key0 / page];                                                                \
+            const bf16* vbase = vc + ((size_t)pg * nkv + kvh) * D * page + (key0 % page);                  \
+            _Pragma("unroll") for (int db = 0; db < D16; ++db)                                             \
+                VF_[db] = *reinterpret_cast<const uint4*>(vbase + (size_t)(db * 16 + r) * page);           \
+        }                                                                                                  \
+    }
+#define ATT_COMPUTE(KF_, VF_, STEP_)                                                                       \
+    {                                                                                                      \
+        const int kb_ = split * span + (STEP_) * ATT_STEP + wave * 32;                                     \
+        const int kbeg_ = kb_ > c_begin ? kb_ : c_begin, kend_ = kb_ + 32 < c_end ? kb_ + 32 : c_end;     \
+        if (kbeg_ < kend_) {   /* wave-uniform */                                                          \
+            f32x4 s[2];                                                                                    \
+            _Pragma("unroll") for (int tau = 0; tau < 2; ++tau) {                                          \
+                s[tau] = f32x4{0.f, 0.f, 0.f, 0.f};                                                        \
+                _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
+                    const int dofs = ks * 32 + qg * 8;                                                     \
+                    s[tau] = mfma16(dofs < D ? KF_[tau][ks] : zero4, qf[ks], s[tau]);                      \
+                }                                                                                          \
+            }                                                                                              \
+            /* lane (r, qg) holds, for head column r, keys kb + qg*8 + tau*4 + e */                       \
+            float sv[8];                                                                                   \
+            float mx = NEG_BIG;                                                                            \
+            _Pragma("unroll") for (int tau = 0; tau < 2; ++tau)                                            \
+                _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                            \
+                    const int key = kb_ + qg * 8 + tau * 4 + e;                                            \
+                    const bool ok = key >= kbeg_ && key < kend_;                                           \
+                    const float v = ok ? s[tau][e] * scale_log2e : NEG_BIG;                                \
+                    sv[tau * 4 + e] = v;                                                                   \
+                    mx = fmaxf(mx, v);                                                                     \
+                }                                                                                          \
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));                                                        \
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));                                                        \
+            const float m_new = fmaxf(m, mx);                                                              \
+            const float corr = __builtin_amdgcn_exp2f(m - m_new);                                          \
+            float pe[8];                                                                                   \
+            float rs = 0.f;                                                                                \
+            _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                                \
+                pe[j] = (sv[j] > 0.5f * NEG_BIG) ? __builtin_amdgcn_exp2f(sv[j] - m_new) : 0.f;            \
+                rs += pe[j];                                                                               \
+            }                                                                                              \
+            rs += __shfl_xor(rs, 16, 64);                                                                  \
+            rs += __shfl_xor(rs, 32, 64);                                                                  \
+            lsum = lsum * corr + rs;                                                                       \
+            m = m_new;                                                                                     \
+            uint4 pf;                                                                                      \
+            pf.x = pack_bf16x2(pe[0], pe[1]);                                                              \
+            pf.y = pack_bf16x2(pe[2], pe[3]);                                                              \
+            pf.z = pack_bf16x2(pe[4], pe[5]);                                                              \
+            pf.w = pack_bf16x2(pe[6], pe[7]);                                                              \
+            const int key0 = kb_ + qg * 8;                                                                 \
+            const bool vok = key0 < kend_ && key0 + 8 > kbeg_;  /* else the loaded values are another group's */ \
+            _Pragma("unroll") for (int db = 0; db < D16; ++db) {                                           \
+                _Pragma("unroll") for (int e = 0; e < 4; ++e) acc[db][e] *= corr;                          \
+                acc[db] = mfma16(vok ? VF_[db] : zero4, pf, acc[db]);                                      \
+            }                                                                                              \
+        }                                                                                                  \
+    }
+    uint4 kfa[2][KS], vfa[D16], kfb[2][KS], vfb[D16];
+    ATT_LOAD(kfa, vfa, first_step)
+    for (int st = first_step; st <= last_step; st += 2) {
+        if (st + 1 <= last_step) ATT_LOAD(kfb, vfb, st + 1)
+        __builtin_amdgcn_sched_barrier(0);
+        ATT_COMPUTE(kfa, vfa, st)
+        if (st + 1 > last_step) break;
+        if (st + 2 <= last_step) ATT_LOAD(kfa, vfa, st + 2)
+        __builtin_amdgcn_sched_barrier(0);
+        ATT_COMPUTE(kfb, vfb, st + 1)
+    }
+#undef ATT_LOAD
+#undef ATT_COMPUTE
     // ---- merge the four waves; acc[db][e] is dim db*16 + qg*4 + e of head column r
 #pragma unroll
     for (int db = 0; db < D16; ++db) *reinterpret_cast<f32x4*>(&sm_acc[wave][db][lane][0]) = acc[db];
@@ -238,13 +235,13 @@ attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __re
 __global__ void __launch_bounds__(64)
 attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
                   const int* __restrict__ pos, const int* __restrict__ rows, int nh, int D, int out_stride,
-                  int window, int nsplit) {
+                  int window, int nsplit, int span) {
     __shared__ float wsm[64];
     const int t = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
     const int h = blockIdx.y, lane = threadIdx.x;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    const int s_lo = lo / ATT_CHUNK, s_hi = p / ATT_CHUNK;
+    const int s_lo = lo / span, s_hi = p / span;
     const size_t base = ((size_t)t * nh + h) * nsplit;
     float o[4] = {0.f, 0.f, 0.f, 0.f};  // dims lane, lane+64, ... (D <= 256)
     float M = NEG_BIG, L = 0.f;
@@ -781,12 +778,12 @@ extern "C" int ilm_attn_tile(void* out, const void* q, const void* kc, const voi
 }
 
 
-extern "C" int ilm_attn_mfma_chunk() { return ATT_CHUNK; }
+extern "C" int ilm_attn_mfma_step() { return ATT_STEP; }
 
 extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q, const void* kc,
                              const void* vc, const void* block_tables, const void* seg, const void* pos,
                              const void* rows, int T_, int nh, int nkv, int d, int page, int max_blocks,
-                             int q_stride, int out_stride, float scale, int window, int nsplit,
+                             int q_stride, int out_stride, float scale, int window, int nsplit, int span,
                              hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_mfma: bad head counts nh=%d nkv=%d", nh, nkv);
     ILM_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attn_mfma: head size %d is not a multiple of 16 up to 128", d);
@@ -794,6 +791,7 @@ extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q
     ILM_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0 && ((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 7) == 0,
                 "attn_mfma: q and out rows must be 16-byte / 8-byte aligned");
     ILM_REQUIRE(nsplit >= 1 && (nsplit == 1 || (ws_acc != nullptr && ws_ml != nullptr)), "attn_mfma: workspace missing");
+    ILM_REQUIRE(span > 0 && span % ATT_STEP == 0, "attn_mfma: chunk of %d keys is no multiple of %d", span, ATT_STEP);
     const int G = nh / nkv, HG = (G + 15) / 16;
     ILM_REQUIRE(nkv * HG <= 65535 && nsplit <= 65535, "attn_mfma: grid too large");
     dim3 grid(T_, nkv * HG, nsplit);
@@ -803,7 +801,7 @@ extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q
         attn_mfma_kernel<D16><<<grid, ATT_WAVES * 64, 0, stream>>>(                                            \
             (bf16*)out, (float*)ws_acc, (float*)ws_ml, (const bf16*)q, (const bf16*)kc, (const bf16*)vc,      \
             (const int*)block_tables, (const int*)seg, (const int*)pos, (const int*)rows, nh, nkv, page,      \
-            max_blocks, q_stride, out_stride, sl2, window, nsplit);                                            \
+            max_blocks, q_stride, out_stride, sl2, window, nsplit, span);                                      \
         break
     switch (d / 16) {
         AM_CASE(1); AM_CASE(2); AM_CASE(3); AM_CASE(4); AM_CASE(5); AM_CASE(6); AM_CASE(7); AM_CASE(8);
@@ -814,7 +812,7 @@ extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q
     if (nsplit > 1) {
         dim3 g2(T_, nh);
         attn_merge_kernel<<<g2, 64, 0, stream>>>((bf16*)out, (const float*)ws_acc, (const float*)ws_ml, (const int*)pos,
-                                                 (const int*)rows, nh, d, out_stride, window, nsplit);
+                                                 (const int*)rows, nh, d, out_stride, window, nsplit, span);
         ILM_LAUNCH_CHECK("attn_merge");
     }
     return 0;

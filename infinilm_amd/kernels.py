@@ -18,7 +18,8 @@ F32 = torch.float32
 BF16 = torch.bfloat16
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 ATT_TILE_TOKENS = 8  # tokens per tile of the prompt-portion attention kernel (ilm_attn_tile_tokens())
-ATT_CHUNK = 256  # keys per chunk of the matrix-core attention kernel (ilm_attn_mfma_chunk())
+ATT_STEP = 128  # keys a workgroup of the chunked attention takes in one step (ilm_attn_mfma_step())
+ATT_MAX_CHUNKS = 64  # most chunks a context is cut into (the merge kernel walks them one after the other)
 # INFINILM_AMD_BASIC=1 runs the plain kernels everywhere (for telling a kernel's fault from the engine's)
 FORCE_BASIC = os.environ.get("INFINILM_AMD_BASIC", "0") == "1"
 SKINNY_VARIANT = int(os.environ.get("INFINILM_AMD_SKINNY_VARIANT", "0"))  # 0: the kernel chooses
@@ -342,6 +343,28 @@ def swiglu_gemm(gate_up: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
     return parts
 
 
+_NUM_CUS: dict = {}
+
+
+def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple:
+    """(keys a chunk, chunks) of the chunked single-token attention for `pairs` = tokens x head groups.
+
+    Enough chunks that the launch has about four workgroups a compute unit (few tokens: short
+    chunks, latency counts; many tokens: long chunks, fewer partial results to write and merge), at
+    most ATT_MAX_CHUNKS.  The length is first rounded up the way the step function rounds its graphs'
+    block tables (pages: 4, 8, 16, ...), so that an eager step and a replayed one cut alike."""
+    pages = 4
+    while pages * page < max_total_len:
+        pages *= 2
+    bound = pages * page
+    cus = _NUM_CUS.get(device)
+    if cus is None:
+        cus = _NUM_CUS[device] = torch.cuda.get_device_properties(device).multi_processor_count
+    wanted = max(1, min(-(-4 * cus // max(pairs, 1)), ATT_MAX_CHUNKS, -(-bound // ATT_STEP)))
+    span = -(-bound // (wanted * ATT_STEP)) * ATT_STEP
+    return span, -(-max_total_len // span)
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int,
                     scale: float, window: int = 0, max_total_len: Optional[int] = None,
@@ -382,7 +405,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 return out
             _i32(single_rows, "single_rows")
             rows, n_single = single_rows, single_rows.numel()
-        nsplit = max(1, -(-int(max_total_len) // ATT_CHUNK))
+        span, nsplit = attention_chunks(int(max_total_len), page, n_single * nkv * (-(-(nh // nkv) // 16)), q.device)
         ws_acc = ws_ml = None
         if nsplit > 1:
             ws_acc = torch.empty((T * nh * nsplit * d,), dtype=F32, device=q.device)
@@ -390,7 +413,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _run("ilm_attn_mfma", out.data_ptr(), _ptr(ws_acc), _ptr(ws_ml), q.data_ptr(), k_cache.data_ptr(),
              v_cache.data_ptr(), block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), _ptr(rows),
              n_single, nh, nkv, d, page, block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window),
-             nsplit, _stream())
+             nsplit, span, _stream())
         return out
     _run("ilm_attn_basic", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
          seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d, page, block_tables.shape[1],

@@ -333,8 +333,22 @@ def test_attention_bfloat16_with_a_moving_maximum(K, ramp):
     _close(out, want, 1.2e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,page,n", [(8, 8, 64, 16, 40), (32, 2, 128, 64, 150), (4, 1, 32, 16, 120)])
+def test_attention_bfloat16_many_single_tokens(K, nh, nkv, d, page, n):
+    """Many decoded tokens in one launch: the chunks get long (several 128-key steps a workgroup,
+    loads a step ahead), contexts from one key to a thousand."""
+    g = torch.Generator().manual_seed(n)
+    lens = torch.randint(1, 1000, (n,), generator=g).tolist()
+    lens[0], lens[1], lens[2] = 1, 1000, 129
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=lens, qlens=[1] * n, seed=n)
+    _close(out, want, 1.2e-2)
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=lens, qlens=[1] * n, seed=n + 1, window=200)
+    _close(out, want, 1.2e-2)
+
+
 def test_attention_does_not_depend_on_the_batch(K):
-    """The same token alone and inside a larger batch gives the same bits (bfloat16 kernel)."""
+    """The same token alone and inside a larger batch gives the same bits (bfloat16 kernel), as long
+    as both launches cut the context into chunks of the same length (few tokens: always 128 keys)."""
     nh, nkv, d, page = 8, 2, 64, 16
     out_a, _ = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[300], qlens=[1], seed=0)
     out_b, _ = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[300, 50, 700], qlens=[1, 50, 2], seed=0)
