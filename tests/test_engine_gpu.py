@@ -290,6 +290,51 @@ def test_kernel_timers_and_engine_counters(models):
     llm.close()
 
 
+class _ToyTokenizer:
+    """Words 'w<id>' separated by blanks: enough of a tokenizer's face for the entry point."""
+    chat_template = "toy"
+
+    def encode(self, text, add_special_tokens=False):
+        return [int(w[1:]) for w in text.split()]
+
+    def decode(self, ids, skip_special_tokens=True):
+        return " ".join(f"w{i}" for i in ids)
+
+    def apply_chat_template(self, messages, tokenize=False, add_generation_prompt=True):
+        return " ".join(m["content"] for m in messages) + (" w1" if add_generation_prompt else "")
+
+
+def test_text_prompts_chat_and_stops(models):
+    """Text in and out through a tokenizer object; chat; a stop string cuts the text and ends the
+    request; a stop token id ends it; ignore_eos runs on."""
+    from infinilm_amd import LLM, SamplingParams
+    from infinilm_amd.engine.request import FinishReason
+
+    cfg, d, W = models[("A", "float32")]
+    llm = LLM(d, dtype="float32", num_blocks=32, block_size=16, max_batch_size=4, tokenizer=_ToyTokenizer())
+    prompt = random_tokens(cfg, 6, 77)
+    want = P.plain_greedy(cfg, W, prompt, 10)
+    text = " ".join(f"w{i}" for i in prompt)
+    sp = SamplingParams(top_k=1, max_tokens=10, ignore_eos=True)
+    out = llm.generate([text], sampling_params=sp)[0]
+    assert out.outputs[0].token_ids == want and out.outputs[0].text == " ".join(f"w{i}" for i in want)
+    assert out.prompt == text and out.finish_reason == FinishReason.LENGTH
+    # chat: the template's text is encoded; here it appends the token 1 to the user's words
+    chat = llm.chat([{"role": "user", "content": text}], sampling_params=sp)[0]
+    assert chat.outputs[0].token_ids == P.plain_greedy(cfg, W, prompt + [1], 10)
+    # a stop string: the text ends before it, the request is finished with that reason
+    stop = f"w{want[3]} w{want[4]}"
+    cut = llm.generate([text], sampling_params=SamplingParams(top_k=1, max_tokens=10, stop=[stop]))[0]
+    assert cut.finish_reason == FinishReason.STOP_STRING
+    assert cut.outputs[0].text == " ".join(f"w{i}" for i in want[:3]) + " " and len(cut.outputs[0].token_ids) == 5
+    # a stop token id
+    st = llm.generate([text], sampling_params=SamplingParams(top_k=1, max_tokens=10, stop_token_ids=[want[2]]))[0]
+    first = want.index(want[2])
+    assert st.finish_reason == FinishReason.STOP and st.outputs[0].token_ids == want[:first + 1]
+    assert llm.engine.stats()["cache"]["running"] == 0 and llm.engine.stats()["cache"]["groups"][0]["free"] == 32
+    llm.close()
+
+
 def test_benchmark_example(models):
     """examples/bench.py: the case grid in order of cache size, one JSON line a case."""
     import json
