@@ -145,7 +145,7 @@ def plain_apply_rope(x: torch.Tensor, pos: torch.Tensor, cos: torch.Tensor, sin:
 
 
 def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
-                    window: int = 0) -> torch.Tensor:
+                    window: int = 0, first_row: int = 0) -> torch.Tensor:
     """Causal grouped-query attention of one whole sequence.
 
     q [T, nh, d], k/v [T, nkv, d] -> [T, nh, d].  Query head h uses KV head h // (nh/nkv)
@@ -153,18 +153,20 @@ def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: fl
     csrc/layers/attention/backends/static_attn.cpp:82-99; scale = 1/sqrt(head_dim):
     csrc/layers/attention/attention.cpp:41.  `window` > 0 keeps only the last `window` keys
     (this architecture never sets it; the engine's parts take it as a parameter).
+    `first_row` > 0 computes (and returns) only the query rows from there on.
     """
     T, nh, d = q.shape
     nkv = k.shape[1]
     g = nh // nkv
-    out = torch.empty_like(q)
+    rows = torch.arange(first_row, T)
+    out = torch.empty_like(q[first_row:])
     i = torch.arange(T)
-    mask = i[None, :] <= i[:, None]
+    mask = i[None, :] <= rows[:, None]
     if window > 0:
-        mask &= i[None, :] > (i[:, None] - window)
+        mask &= i[None, :] > (rows[:, None] - window)
     for h in range(nh):
         kh = h // g
-        s = (q[:, h, :] @ k[:, kh, :].T) * scale
+        s = (q[first_row:, h, :] @ k[:, kh, :].T) * scale
         s = s.masked_fill(~mask, float("-inf"))
         p = torch.softmax(s, dim=-1)
         out[:, h, :] = p @ v[:, kh, :]

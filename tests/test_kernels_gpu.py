@@ -291,8 +291,8 @@ def _attention_case(K, dtype, nh, nkv, d, page, lens, qlens, window=0, seed=0, s
                             max_total_len=max(lens), **extra)
     want = []
     for i, (n, ql) in enumerate(zip(lens, qlens)):
-        full = P.plain_attention(qs[i].to(F64), ks[i].to(F64), vs[i].to(F64), 1 / math.sqrt(d), window)
-        want.append(full[n - ql:].reshape(ql, nh * d))
+        last = P.plain_attention(qs[i].to(F64), ks[i].to(F64), vs[i].to(F64), 1 / math.sqrt(d), window, first_row=n - ql)
+        want.append(last.reshape(ql, nh * d))
     return out, torch.cat(want)
 
 
@@ -343,6 +343,15 @@ def test_attention_bfloat16_many_single_tokens(K, nh, nkv, d, page, n):
     out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=lens, qlens=[1] * n, seed=n)
     _close(out, want, 1.2e-2)
     out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=lens, qlens=[1] * n, seed=n + 1, window=200)
+    _close(out, want, 1.2e-2)
+
+
+def test_attention_bfloat16_with_a_block_table_beyond_lds(K):
+    """33,000 keys in pages of 16: more block-table entries than the tile kernel keeps in LDS, and
+    the most chunks the single-token kernel cuts a context into."""
+    out, want = _attention_case(K, torch.bfloat16, 4, 2, 64, 16, lens=[33000, 50], qlens=[11, 1], seed=41)
+    _close(out, want, 1.2e-2)
+    out, want = _attention_case(K, torch.bfloat16, 4, 2, 64, 16, lens=[33000, 70], qlens=[1, 1], seed=42)
     _close(out, want, 1.2e-2)
 
 
