@@ -21,7 +21,7 @@ def main(argv=None) -> int:
     logging.basicConfig(level=getattr(logging, cfg.log_level.upper(), logging.INFO))
     model = LLM(model_path=os.path.expanduser(cfg.model), device=cfg.get_device_str(cfg.device, cfg.device_id),
                 dtype=cfg.dtype, max_batch_size=max(cfg.batch_size, 1), max_tokens=cfg.max_new_tokens,
-                num_blocks=cfg.num_blocks, block_size=cfg.block_size, temperature=cfg.temperature, top_k=cfg.top_k,
+                num_blocks=cfg.num_blocks or None, block_size=cfg.block_size, temperature=cfg.temperature, top_k=cfg.top_k,
                 top_p=cfg.top_p, enable_graph=cfg.enable_graph, attn_backend=cfg.attn,
                 skip_load=cfg.skip_load or cfg.random_weights, max_num_batched_tokens=cfg.max_num_batched_tokens,
                 chunk_size=cfg.chunk_size, admission=cfg.admission, seed=cfg.seed)

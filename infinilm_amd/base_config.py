@@ -28,7 +28,7 @@ class BaseConfig:
         ap.add_argument("--temperature", type=float, default=1.0)
         ap.add_argument("--enable-paged-attn", action="store_true", help="accepted; the cache is always paged")
         ap.add_argument("--attn", type=str, default="default", choices=["default", "paged-attn"])
-        ap.add_argument("--num-blocks", type=int, default=512)
+        ap.add_argument("--num-blocks", type=int, default=512, help="pages of the cache pool; 0: what the free device memory holds")
         ap.add_argument("--block-size", type=int, default=256)
         ap.add_argument("--max-batch-size", type=int, default=8)
         ap.add_argument("--max-num-batched-tokens", type=int, default=None)

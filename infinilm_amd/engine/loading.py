@@ -55,8 +55,28 @@ def load_model(model_dir: str, dtype=None, device="cuda:0") -> CausalLM:
     return model
 
 
-def make_runner(model: CausalLM, num_pages: int, page_size: int, max_requests: int,
+def pages_that_fit(model: CausalLM, page_size: int, memory_fraction: float = 0.9, reserve_bytes: int = 4 << 30) -> int:
+    """Pages per group that `memory_fraction` of the device's free memory holds (after `reserve_bytes`
+    for activations, graphs and workspaces), for `num_pages=None`: the cache takes what the weights
+    leave, on a 288 GB part some hundred thousand tokens for a model of this size."""
+    from ..cache.needs import PagedKV
+    elem = torch.empty((), dtype=model.dtype).element_size()
+    per_page = sum(2 * n.num_kv_heads * n.head_dim * page_size * elem for n in model.cache_needs if isinstance(n, PagedKV))
+    if per_page == 0:
+        return 1
+    free, _ = torch.cuda.mem_get_info(model.device)
+    usable = int(free * memory_fraction) - reserve_bytes
+    if usable < per_page:
+        raise RuntimeError(f"no room for a cache: {free / 2**30:.1f} GiB free on {model.device}, a page of every layer "
+                           f"takes {per_page / 2**20:.1f} MiB")
+    return usable // per_page
+
+
+def make_runner(model: CausalLM, num_pages: Optional[int], page_size: int, max_requests: int,
                 enable_graph: bool = False) -> StepRunner:
+    """`num_pages=None`: as many pages as fit into the free device memory (see `pages_that_fit`)."""
+    if num_pages is None:
+        num_pages = pages_that_fit(model, page_size)
     cache = CacheManager(model.cache_needs, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
                          dtype=model.dtype, device=model.device)
     return StepRunner(model, cache, enable_graph=enable_graph)

@@ -35,14 +35,14 @@ class LLM:
     dtype           "bfloat16" | "float32" | None (config.json's); float32 is true 32-bit throughout
     max_batch_size  most requests in flight
     max_tokens      default cap of generated tokens per request
-    num_blocks / block_size   pages of the cache pool / tokens a page
+    num_blocks / block_size   pages of the cache pool (None: what the free device memory holds) / tokens a page
     temperature / top_p / top_k   defaults of requests that bring no SamplingParams
     max_num_batched_tokens / chunk_size   token budget of a step / longest portion of a prompt
     admission       "optimistic" (preempt when pages run out) | "reserve_full" (the reference's check)
     """
 
     def __init__(self, model_path, device: str = "cuda", dtype: Optional[str] = None, cache_type: str = "paged",
-                 max_batch_size: int = 16, max_tokens: int = 4096, num_blocks: int = 512, block_size: int = 256,
+                 max_batch_size: int = 16, max_tokens: int = 4096, num_blocks: Optional[int] = 512, block_size: int = 256,
                  max_cache_len: Optional[int] = None, temperature: float = 1.0, top_p: float = 0.8, top_k: int = 1,
                  enable_graph: bool = False, attn_backend: str = "default", skip_load: bool = False,
                  enable_prefix_caching: bool = False, max_num_batched_tokens: Optional[int] = None,
