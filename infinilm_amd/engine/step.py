@@ -17,6 +17,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
+from .. import kernels
 from ..cache import CacheManager
 
 
@@ -136,7 +137,7 @@ class StepRunner:
         n_want = sum(len(e.want) for e in entries)
 
         # attention work lists: runs of up to TILE consecutive tokens of a request, and single tokens
-        TILE = 8
+        TILE = kernels.ATT_TILE_TOKENS
         tiles: List[int] = []
         singles: List[int] = []
         for i in range(R):

@@ -32,6 +32,14 @@ def _close(got, want, tol):
     assert err < tol, f"error {err:.3e} above {tol:.1e}"
 
 
+def test_constants_mirrored_in_python_equal_the_library(K):
+    from infinilm_amd.csrc import lib
+    L = lib.load()
+    assert L.ilm_attn_tile_tokens() == K.ATT_TILE_TOKENS
+    assert L.ilm_attn_mfma_step() == K.ATT_STEP
+    assert L.ilm_gemm_ksplit_max_k(1) == K.KSPLIT_SPAN
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_embed(K, dtype):
     table = _rand((331, 80), 1, dtype)
