@@ -224,9 +224,17 @@ extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void
         gemm_skinny_resident_kernel<WV, KS, TC><<<grid, WV * 64, 0, stream>>>(                              \
             (TC*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha, ntiles); \
     }
+        // measured on MI355X at K = 4096: 8 waves of 16 k-steps (more loads in flight a wave) win where the
+        // tiles are at most one a compute unit (o projection, 9.1 against 10.2 us) or many (gate/up 47.8
+        // against 50.0 us, the head), 16 waves of 8 where they are a few more than the compute units
+        // (q/k/v).  Two tiles in flight instead of one changed nothing.  INFINILM_AMD_SKINNY_FAT=0: always 16 x 8.
+        static int fat = -1;
+        if (fat < 0) { const char* e = getenv("INFINILM_AMD_SKINNY_FAT"); fat = e ? atoi(e) : 1; }
+        const bool fat_waves = fat && ksteps > 8 * 8 && ksteps <= 8 * 16 && (ntiles <= num_cus() || ntiles >= 4 * num_cus());
 #define SR_DISPATCH(TC)                                   \
     if (ksteps <= 8 * 4) SR_CASE(8, 4, TC)                \
     else if (ksteps <= 8 * 8) SR_CASE(8, 8, TC)           \
+    else if (fat_waves) SR_CASE(8, 16, TC)                \
     else if (ksteps <= 16 * 8) SR_CASE(16, 8, TC)         \
     else SR_CASE(16, 16, TC)
         if (out_dtype == ILM_DTYPE_BF16) { SR_DISPATCH(bf16) } else { SR_DISPATCH(float) }
