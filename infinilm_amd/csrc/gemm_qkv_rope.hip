@@ -3,12 +3,14 @@
 // two between the norm and the attention.
 //
 // The product is the resident few-rows one (X fragments in registers, W streamed once on
-// v_mfma_f32_16x16x32_bf16, K split over the waves and reduced through LDS).  A workgroup takes
-// units of two 16-row tiles of W, rows [hs*d + j*16, +16) and [hs*d + d/2 + j*16, +16) of head slot
-// hs: the two halves of 16 rotation pairs.  The thread that reduces output (m, n) of the first
-// tile also reduces (m, n) of the second, so it holds a pair in registers, rotates it by the
-// token's position and stores it: q into the output rows, k into the token's cache slot; v tiles
-// take the same path without rotation into the transposed value cache.
+// v_mfma_f32_16x16x32_bf16, K split over the waves and reduced through LDS).  Rows i and i + d/2 of
+// a head slot (q head, k head or v head) form a pair; a workgroup takes a run of up to 16
+// consecutive pairs and multiplies two 16-row tiles of W: the pairs' first rows and their second
+// rows.  The thread that reduces output (m, n) of the first tile also reduces (m, n) of the
+// second, so it holds a pair in registers, rotates it by the token's position and stores it: q
+// into the output rows, k into the token's cache slot; v pairs take the same path without
+// rotation into the transposed value cache.  The run length is chosen so that every compute unit
+// gets one run (9 pairs = 18 rows at the 8B shape: no second round for a few leftover tiles).
 // Needs the whole head rotated (rotary dim = head dim) and head dims in steps of 32.
 #include "common.h"
 
@@ -28,14 +30,14 @@ gemm_qkv_rope_kernel(bf16* __restrict__ Q, const bf16* __restrict__ X, const bf1
                      const bf16* __restrict__ bias, int M, int K, int lda, int ldw, int ldq,
                      const int* __restrict__ pos, const float* __restrict__ cosT, const float* __restrict__ sinT,
                      bf16* __restrict__ kc, bf16* __restrict__ vc, const int* __restrict__ slots, int nh, int nkv,
-                     int d, int page, int n_units) {
+                     int d, int page, int n_units, int pairs_per_unit) {
     __shared__ float part[2][WAVES][64][4];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, q = lane >> 4;
     const int s0 = wave * KSTEPS;
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     const int k8_last = (K >> 3) - 1;
-    const int half = d >> 1, upt = d >> 5;   // units per head slot
+    const int half = d >> 1;
     uint4 xf[KSTEPS];
     int k8c[KSTEPS];
     {
@@ -48,26 +50,34 @@ gemm_qkv_rope_kernel(bf16* __restrict__ Q, const bf16* __restrict__ X, const bf1
             xf[u] = (k8 <= k8_last && r < M) ? v : zero;   // zero fragments make the clamped W loads harmless
         }
     }
-    // first W row of tile `half_idx` (0, 1) of unit u
-    auto tile_row = [&](int u, int half_idx) -> int { return (u / upt) * d + (u % upt) * 16 + half_idx * half; };
+    // pair p: rows hs*d + i and hs*d + i + d/2 with hs = p / (d/2), i = p % (d/2)
+    const int total_pairs = (nh + 2 * nkv) * half;
+    auto first_row = [&](int pair) -> int { return (pair / half) * d + pair % half; };
+    // this lane's W row of a unit's tile (0: first rows, 1: second rows); lanes beyond the run repeat its last pair
+    auto tile_row = [&](int u, int half_idx) -> int {
+        const int p0 = u * pairs_per_unit;
+        const int np = total_pairs - p0 < pairs_per_unit ? total_pairs - p0 : pairs_per_unit;
+        return first_row(p0 + (r < np ? r : np - 1)) + half_idx * half;
+    };
     uint4 a[KSTEPS];
     int unit = blockIdx.x;
     if (unit < n_units) {
-        const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)(tile_row(unit, 0) + r) * ldw);
+        const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)tile_row(unit, 0) * ldw);
 #pragma unroll
         for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
     }
-    // the epilogue thread's output: row m, column nl of a tile
+    // the epilogue thread's output: row m, pair slot nl of the run
     const int et = threadIdx.x < 256 ? threadIdx.x : 0;
     const int e = et & 3, l = et >> 2;
     const int m = l & 15, nl = (l >> 4) * 4 + e;
-    const bool writer = threadIdx.x < 256 && m < M;
-    const int p_m = writer ? pos[m] : 0;
-    const int slot = (writer && slots != nullptr) ? slots[m] : -1;
+    const bool row_writer = threadIdx.x < 256 && m < M;
+    const int p_m = row_writer ? pos[m] : 0;
+    const int slot = (row_writer && slots != nullptr) ? slots[m] : -1;
     int buf = 0;
     for (; unit < n_units; unit += gridDim.x) {
-        const int hs = unit / upt, j = unit % upt;
-        const int i0 = j * 16 + nl;   // this thread's dim within the first half of the head
+        const int pair = unit * pairs_per_unit + nl;
+        const bool writer = row_writer && nl < pairs_per_unit && pair < total_pairs;
+        const int hs = writer ? pair / half : 0, i0 = writer ? pair % half : 0;   // head slot, dim within its first half
         float cs = 1.f, sn = 0.f;
         if (writer && hs < nh + nkv) {   // on their way while the products run
             cs = cosT[(size_t)p_m * half + i0];
@@ -83,7 +93,7 @@ gemm_qkv_rope_kernel(bf16* __restrict__ Q, const bf16* __restrict__ X, const bf1
             const int nu = hf == 0 ? unit : unit + gridDim.x;
             __builtin_amdgcn_sched_barrier(0);
             if (nu < n_units) {
-                const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)(tile_row(nu, hf == 0 ? 1 : 0) + r) * ldw);
+                const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)tile_row(nu, hf == 0 ? 1 : 0) * ldw);
 #pragma unroll
                 for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
             }
@@ -94,7 +104,7 @@ gemm_qkv_rope_kernel(bf16* __restrict__ Q, const bf16* __restrict__ X, const bf1
             if (threadIdx.x < 256) {
 #pragma unroll
                 for (int w = 0; w < WAVES; ++w) v += part[buf][w][l][e];
-                if (bias != nullptr) v += to_f32(bias[tile_row(unit, hf) + nl]);
+                if (bias != nullptr && writer) v += to_f32(bias[hs * d + i0 + hf * half]);
             }
             val[hf] = qr_round(v);
             buf ^= 1;  // the other buffer is free: its readers passed the barrier above one tile ago
@@ -145,15 +155,19 @@ extern "C" int ilm_gemm_qkv_rope(void* Q, int ldq, const void* X, int lda, const
     ILM_REQUIRE(slots == nullptr || (page > 0 && kc != nullptr && vc != nullptr), "gemm_qkv_rope: cache missing");
     const int ksteps = (K + 31) / 32;
     ILM_REQUIRE(ksteps <= 16 * 16, "gemm_qkv_rope: K=%d is beyond 8192", K);
-    const int n_units = (nh + 2 * nkv) * (d / 32);
+    // runs of pairs: one a compute unit where that gives at most 16 pairs a run, else runs of 16 in rounds
+    const int total_pairs = (nh + 2 * nkv) * (d / 2);
 #define QR_CASE(WV, KS)                                                                                        \
     {                                                                                                          \
         const int cap = qr_num_cus() * (WV == 16 ? 1 : 2);                                                     \
+        int ppu = (total_pairs + cap - 1) / cap;                                                               \
+        if (ppu > 16) ppu = 16;                                                                                \
+        const int n_units = (total_pairs + ppu - 1) / ppu;                                                     \
         const int grid = n_units < cap ? n_units : cap;                                                        \
         gemm_qkv_rope_kernel<WV, KS><<<grid, WV * 64, 0, stream>>>(                                            \
             (bf16*)Q, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, K, lda, ldw, ldq, (const int*)pos, \
             (const float*)cosT, (const float*)sinT, (bf16*)kc, (bf16*)vc, (const int*)slots, nh, nkv, d, page, \
-            n_units);                                                                                          \
+            n_units, ppu);                                                                                     \
     }
     if (ksteps <= 8 * 4) QR_CASE(8, 4)
     else if (ksteps <= 8 * 8) QR_CASE(8, 8)
