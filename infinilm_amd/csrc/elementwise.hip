@@ -93,17 +93,27 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __res
             v[it][4] = r1.x; v[it][5] = r1.y; v[it][6] = r1.z; v[it][7] = r1.w;
             if (h != nullptr) {
                 float hs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                for (int p = 0; p < parts; ++p) {   // parts of a K-split product, summed in order
-                    HT hv[8];
-                    const HT* hp = h + p * pstride + base + j;
-                    if (sizeof(HT) == 2) {
-                        *reinterpret_cast<uint4*>(hv) = *reinterpret_cast<const uint4*>(hp);
-                    } else {
-                        *reinterpret_cast<float4*>(hv) = *reinterpret_cast<const float4*>(hp);
-                        *reinterpret_cast<float4*>(hv + 4) = *reinterpret_cast<const float4*>(hp + 4);
+                // parts of a K-split product, summed in order; loaded four at a time, so that their
+                // latencies overlap (a product of many rows comes in up to 16 parts)
+                for (int p0 = 0; p0 < parts; p0 += 4) {
+                    HT hv[4][8];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int p = p0 + u < parts ? p0 + u : parts - 1;
+                        const HT* hp = h + p * pstride + base + j;
+                        if (sizeof(HT) == 2) {
+                            *reinterpret_cast<uint4*>(hv[u]) = *reinterpret_cast<const uint4*>(hp);
+                        } else {
+                            *reinterpret_cast<float4*>(hv[u]) = *reinterpret_cast<const float4*>(hp);
+                            *reinterpret_cast<float4*>(hv[u] + 4) = *reinterpret_cast<const float4*>(hp + 4);
+                        }
                     }
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) hs[e] += to_f32(hv[e]);
+                    for (int u = 0; u < 4; ++u)
+                        if (p0 + u < parts) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) hs[e] += to_f32(hv[u][e]);
+                        }
                 }
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[it][e] += alpha * hs[e];

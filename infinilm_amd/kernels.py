@@ -283,6 +283,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     aligned = K % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 \
         and w.data_ptr() % 16 == 0
     plain = bias is None and alpha == 1.0
+    # 65 to 128 rows on their way into the residual sum: split over K, where the vendor library leaves the
+    # chip idle (measured at the 8B shapes: down projection 68 -> 36 us at 96 rows, 81 -> 39 at 128; o
+    # projection 22 -> 17 and 25 -> 19; up to 64 rows the library and a one-part sum are as fast)
+    if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS:
+        return _gemm_mid(a, w, K, False)
     if fast and aligned and plain and allow_parts and out is None and M <= 16 and K > 2 * KSPLIT_SPAN and USE_KSPLIT:
         kb = -(-K // KSPLIT_SPAN)
         parts = torch.empty((kb, M, N), dtype=F32, device=a.device)
@@ -325,13 +330,34 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     return out
 
 
+MID_MAX_ROWS = int(os.environ.get("INFINILM_AMD_MID_ROWS", "128"))  # 16: above 16 rows always the library
+MID_TARGET_WGS = int(os.environ.get("INFINILM_AMD_MID_WGS", "512"))
+
+
+def _gemm_mid(x: torch.Tensor, w: torch.Tensor, K: int, act: bool) -> torch.Tensor:
+    """17 to 128 rows, result in float32 parts [P, M, N] split over K (see gemm_mid.hip); `act`: x holds
+    rows [gate | up] and the product takes silu(gate) * up."""
+    M, N = x.shape[0], w.shape[0]
+    n_tiles = -(-N // 128)
+    kb = max(1, min(-(-MID_TARGET_WGS // n_tiles), K // 512 or 1))
+    kspan = -(-K // (kb * 128)) * 128
+    kb = -(-K // kspan)
+    parts = torch.empty((kb, M, N), dtype=F32, device=x.device)
+    _run("ilm_gemm_mid", parts.data_ptr(), N, M * N, kb, kspan, w.data_ptr(), w.stride(0), M, N, K, x.data_ptr(),
+         x.stride(0), 1 if act else 0, _stream())
+    return parts
+
+
 def swiglu_gemm(gate_up: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
     """(silu(gate) * up) w^T for at most 16 rows [gate | up] in bfloat16, in one kernel: float32 parts
     [P, M, N] for add_rmsnorm.  None when the shapes do not fit (the caller then runs the two kernels)."""
     M, two_k = gate_up.shape
     K = two_k // 2
     N = w.shape[0]
-    ok = (gate_up.dtype == BF16 and w.dtype == BF16 and not FORCE_BASIC and USE_KSPLIT and M <= 16 and two_k % 2 == 0
+    # (above 16 rows the activation would be recomputed by every workgroup along N: the separate kernel
+    # and the medium-rows product are faster, 38 against 42 us at 64 rows)
+    ok = (gate_up.dtype == BF16 and w.dtype == BF16 and not FORCE_BASIC and USE_KSPLIT and M <= 16
+          and two_k % 2 == 0
           and w.shape[1] == K and K % 8 == 0 and gate_up.stride(1) == 1 and w.stride(1) == 1 and gate_up.stride(0) % 8 == 0
           and w.stride(0) % 8 == 0 and gate_up.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and gate_up.is_cuda)
     if not ok:

@@ -202,18 +202,23 @@ def test_gemm_bfloat16(K, M, N, K_, out_dtype):
         _close(out, P.plain_linear(a.to(F64), w.to(F64), b.to(F64), 0.5), 1e-5 if out_dtype == torch.float32 else 6e-3)
 
 
-@pytest.mark.parametrize("M,N,K_", [(8, 4096, 16384), (1, 50, 8200), (16, 331, 12296)])
+@pytest.mark.parametrize("M,N,K_", [(8, 4096, 16384), (1, 50, 8200), (16, 331, 12296), (17, 4096, 4096), (64, 4096, 16384),
+                                    (48, 331, 200), (35, 50, 8200), (128, 1030, 1096), (97, 64, 72)])
 def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
     """Few rows and long K: the product comes as float32 parts; add_rmsnorm sums them in order."""
     a, w = _rand((M, K_), 14, torch.bfloat16), _rand((N, K_), 15, torch.bfloat16, 0.05)
     parts = K.gemm(a.to(DEV), w.to(DEV), allow_parts=True)
-    assert parts.dim() == 3 and parts.dtype == torch.float32 and parts.shape[0] == -(-K_ // 4096)
+    if 16 < M <= 64:   # the library serves these; the kernel itself is tested all the same
+        parts = K._gemm_mid(a.to(DEV), w.to(DEV), K_, False)
+    assert parts.dim() == 3 and parts.dtype == torch.float32 and (M > 16 or parts.shape[0] == -(-K_ // 4096))
     want = P.plain_linear(a.to(F64), w.to(F64))
     _close(parts.sum(0), want, 1e-5)
     whole = K.gemm(a.to(DEV), w.to(DEV))
     assert whole.dim() == 2 and whole.dtype == torch.bfloat16
     short = K.gemm(a[:, :256].contiguous().to(DEV), w[:, :256].contiguous().to(DEV), allow_parts=True)
-    assert short.dim() == 2 and short.dtype == torch.float32   # short K: one part, not rounded to bfloat16
+    # short K: one part, not rounded to bfloat16 (more than 64 rows: the medium-rows kernel with its parts;
+    # 17 to 64: the library's bfloat16)
+    assert (short.dtype == torch.float32 and short.dim() == 2) if M <= 16 else (short.dim() == 3 if M > 64 else short.dtype == torch.bfloat16)
     _close(whole, want, 6e-3)
     r = _rand((M, N), 16, scale=2.0)
     nw = _rand((N,), 17, torch.bfloat16) + 1
@@ -224,15 +229,21 @@ def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
     _close(x, P.plain_rmsnorm(want_r, nw.to(F64), 1e-6), 1e-2)
 
 
-@pytest.mark.parametrize("M,I,N", [(8, 16384, 4096), (3, 200, 96), (16, 4104, 50)])
+@pytest.mark.parametrize("M,I,N", [(8, 16384, 4096), (3, 200, 96), (16, 4104, 50), (17, 4104, 50), (40, 8192, 1024),
+                                   (64, 16384, 4096), (33, 96, 331), (128, 1000, 70), (100, 16384, 4096)])
 def test_swiglu_inside_the_down_projection(K, M, I, N):
     gu = _rand((M, 2 * I), 18, torch.bfloat16, 1.5)
     w = _rand((N, I), 19, torch.bfloat16, 0.05)
-    parts = K.swiglu_gemm(gu.to(DEV), w.to(DEV))
-    assert parts is not None and parts.dtype == torch.float32 and parts.shape == (-(-I // 4096), M, N)
+    if M <= 16:
+        parts = K.swiglu_gemm(gu.to(DEV), w.to(DEV))
+    else:   # the medium-rows kernel's variant with the activation on the way into LDS (not on the engine's path)
+        assert K.swiglu_gemm(gu.to(DEV), w.to(DEV)) is None
+        parts = K._gemm_mid(gu.to(DEV), w.to(DEV), I, True)
+    assert parts is not None and parts.dtype == torch.float32 and parts.shape[1:] == (M, N)
+    if M <= 16:
+        assert parts.shape[0] == -(-I // 4096)
     act = P.plain_swiglu(gu.to(F64)[:, :I], gu.to(F64)[:, I:])
     _close(parts.sum(0), P.plain_linear(act, w.to(F64)), 6e-3)   # the activation is rounded to bfloat16 once
-    assert K.swiglu_gemm(_rand((17, 64), 1, torch.bfloat16).to(DEV), _rand((8, 32), 2, torch.bfloat16).to(DEV)) is None
 
 
 def _paged(k, v, page, n_pages, seed, dtype):

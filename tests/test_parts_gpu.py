@@ -124,7 +124,8 @@ def test_attention_part_alone_in_portions(dtype, page, window):
     outs, i = [], 0
     for k in (17, 2, 1, 30, 1, 1, 23):
         b = hz.batch([("r", k)])
-        outs.append(att.forward(x[i:i + k].to(DEV), b, hz.cache.view(0, b, True)))
+        o = att.forward(x[i:i + k].to(DEV), b, hz.cache.view(0, b, True))
+        outs.append(o.sum(0).to(dtype) if o.dim() == 3 else o.to(dtype))   # a branch may come in float32 parts
         hz.commit([("r", k)])
         i += k
     got = torch.cat(outs)
