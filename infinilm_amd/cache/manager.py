@@ -65,6 +65,7 @@ class CacheManager:
             raise CacheError(f"page size must be positive, got {page_size}")
         self.page_size = int(page_size)
         self.max_requests = int(max_requests)
+        self.version = 0   # counts admissions and releases: what was prepared for a set of requests is stale after either
         self.device = torch.device(device)
         self.dtype = dtype
         self.needs = list(needs)
@@ -131,6 +132,7 @@ class CacheManager:
             raise CacheError(f"no state slot free for request {req_id!r} ({self.max_requests} requests at most)")
         r = _Request(tables=[[] for _ in self.groups], state_slot=self._free_slots.pop())
         self.requests[req_id] = r
+        self.version += 1
 
     def has(self, req_id) -> bool:
         return req_id in self.requests
@@ -210,6 +212,7 @@ class CacheManager:
         for g, table in zip(self.groups, r.tables):
             g.pool.give_back([p for p in table if p >= 0])
         self._free_slots.append(r.state_slot)
+        self.version += 1
 
     def check(self) -> None:
         """No page lost, none held twice: the pages in the block tables are exactly the held ones."""

@@ -18,7 +18,7 @@ import numpy as np
 import torch
 
 from .. import kernels
-from ..cache import CacheManager
+from ..cache import CacheError, CacheManager
 
 
 @dataclass
@@ -74,26 +74,39 @@ class StepRunner:
         self._graph_pool = None
         self._graph_seen: Dict = {}      # sizes met in eager steps so far -> how often
         self.graph_after = 2
-        self._pinned: Optional[torch.Tensor] = None
-        self._copy_done: Optional[torch.cuda.Event] = None
+        self._pinned: List[Optional[torch.Tensor]] = [None, None]   # two staging buffers in turn
+        self._copy_done: List[Optional[torch.cuda.Event]] = [None, None]
+        self._stage_turn = 0
+        self._prepared = None            # metadata of the next decode step, built while the device ran this one
         self.steps = 0
         self.tokens = 0
 
     # ---- batch building -----------------------------------------------------------------------
     def _stage(self, n: int) -> torch.Tensor:
-        if self._copy_done is not None:
-            self._copy_done.synchronize()
-        if self._pinned is None or self._pinned.numel() < n:
-            self._pinned = torch.empty((max(n, 4096) * 2,), dtype=torch.int32, pin_memory=self.device.type == "cuda")
-        return self._pinned[:n]
+        """Pinned host memory for a step's metadata; two buffers in turn, each waited for only when its
+        own last copy to the device may still be reading it."""
+        t = self._stage_turn = self._stage_turn ^ 1
+        if self._copy_done[t] is not None:
+            self._copy_done[t].synchronize()
+            self._copy_done[t] = None
+        if self._pinned[t] is None or self._pinned[t].numel() < n:
+            self._pinned[t] = torch.empty((max(n, 4096) * 2,), dtype=torch.int32, pin_memory=self.device.type == "cuda")
+        return self._pinned[t][:n]
+
+    def _copy_to_device(self, dev: torch.Tensor, host: torch.Tensor, turn: int) -> None:
+        dev.copy_(host, non_blocking=True)
+        if self.device.type == "cuda":
+            self._copy_done[turn] = torch.cuda.Event()
+            self._copy_done[turn].record()
 
     def build_batch(self, entries: Sequence[StepEntry], min_blocks: int = 0,
-                    device_buffer: Optional[torch.Tensor] = None) -> StepBatch:
+                    device_buffer: Optional[torch.Tensor] = None, defer_copy: bool = False) -> StepBatch:
         """Reserves pages for every entry and lays the step's metadata out.
 
         `min_blocks` pads the block tables to a fixed width and `device_buffer` receives the
         metadata instead of a fresh tensor: a captured graph reads the same addresses at every
-        replay."""
+        replay.  `defer_copy`: the metadata stays in its staging buffer (`batch.pending_copy`): the
+        caller fills in the token ids and sends it later."""
         cache = self.cache
         V = self.model.spec.vocab_size
         if not entries:
@@ -226,10 +239,8 @@ class StepRunner:
             if device_buffer.numel() < total:
                 raise RuntimeError("the graph's metadata buffer is too small for this step")
             dev = device_buffer[:total]
-        dev.copy_(host, non_blocking=True)
-        if self.device.type == "cuda":
-            self._copy_done = torch.cuda.Event()
-            self._copy_done.record()
+        if not defer_copy:
+            self._copy_to_device(dev, host, self._stage_turn)
 
         def dseg(name):
             o, n = off[name]
@@ -255,6 +266,8 @@ class StepRunner:
         b.h_start_pos = start
         b.h_state_in = np.array(sin, dtype=np.int64)
         b.h_state_out = np.array(sout, dtype=np.int64)
+        if defer_copy:
+            b.pending_copy = (dev, host, self._stage_turn, off["token_ids"][0])
         return b
 
     # ---- the step -----------------------------------------------------------------------------
@@ -315,15 +328,49 @@ class StepRunner:
             self._graphs[key] = (graph, batch, logits, buf)
         else:
             graph, batch, logits, buf = slot
-            fresh = self.build_batch(entries, min_blocks=width, device_buffer=buf)
-            if fresh.T != batch.T or fresh.block_tables[0].shape != batch.block_tables[0].shape:
-                raise RuntimeError("a decode step does not fit the graph captured for its size")
+            ids = tuple(e.req_id for e in entries)
+            prep, self._prepared = self._prepared, None
+            if prep is not None and prep[0] == (key, ids, cache.version) and prep[1] == [cache.length(i) for i in ids]:
+                # built while the device ran the last step: only the token ids are new
+                dev, host, turn, tok_off = prep[2]
+                V = self.model.spec.vocab_size
+                for i, e in enumerate(entries):
+                    if not 0 <= e.tokens[0] < V:
+                        raise ValueError(f"request {e.req_id!r}: token id {e.tokens[0]} is outside the vocabulary of {V}")
+                    host[tok_off + i] = e.tokens[0]
+                self._copy_to_device(dev, host, turn)
+            else:
+                fresh = self.build_batch(entries, min_blocks=width, device_buffer=buf)
+                if fresh.T != batch.T or fresh.block_tables[0].shape != batch.block_tables[0].shape:
+                    raise RuntimeError("a decode step does not fit the graph captured for its size")
         graph.replay()
         for e in entries:
             cache.commit(e.req_id, 1)
         self.steps += 1
         self.tokens += R
+        self._prepare_next_decode(entries)
         return logits
+
+    def _prepare_next_decode(self, entries: Sequence[StepEntry]) -> None:
+        """While the device runs the step just launched: the metadata of the same requests' next decoded
+        tokens (positions, slots, block tables; pages reserved), everything but the token ids.  Used by
+        the next graph step if it is for these requests at these lengths; else dropped (pages
+        reserved here stay with their requests, as after any step that could not run)."""
+        cache = self.cache
+        try:
+            key = self._graph_key(entries)
+            slot = self._graphs.get(key)
+            if slot is None:
+                return
+            ids = tuple(e.req_id for e in entries)
+            lengths = [cache.length(i) for i in ids]
+            if max(lengths) + 1 > self.model.spec.max_positions:
+                return
+            b = self.build_batch([StepEntry(i, [0], [0]) for i in ids], min_blocks=key[1], device_buffer=slot[3],
+                                 defer_copy=True)
+            self._prepared = ((key, ids, cache.version), lengths, b.pending_copy)
+        except (CacheError, ValueError):
+            self._prepared = None   # out of pages for the guess: the real step will say so if it comes
 
     def _graph_buffer_size(self, R: int, width: int) -> int:
         G = len(self.cache.groups)

@@ -101,6 +101,61 @@ def test_graph_replays_equal_eager_steps(models):
     assert len(graph._graphs) >= 2   # the context outgrew the first graph's block-table width
 
 
+def test_graph_steps_with_a_changing_set_of_requests(models):
+    """The next decode step's metadata is prepared while the device runs the current one; it must be
+    dropped when a request ends, another joins, a step of another kind comes between, or the order
+    changes.  Replays must still equal eager steps bit for bit."""
+    from infinilm_amd.engine.loading import load_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+
+    cfg, d, W = models[("C", "bfloat16")]
+    model = load_model(d, "bfloat16", "cuda:0")
+    eager = make_runner(model, num_pages=48, page_size=16, max_requests=6)
+    graph = make_runner(model, num_pages=48, page_size=16, max_requests=6, enable_graph=True)
+    graph.graph_after = 1
+
+    def both(entries):
+        le = eager.step(entries).clone()
+        torch.cuda.synchronize()
+        lg = graph.step(entries)
+        assert torch.equal(le.cpu(), lg.cpu())
+        return le
+
+    def admit(rid, n, seed):
+        for r in (eager, graph):
+            r.cache.admit(rid)
+        both([StepEntry(rid, random_tokens(cfg, n, seed), [n - 1])])
+
+    admit("a", 20, 1), admit("b", 33, 2), admit("c", 7, 3)
+    live = ["a", "b", "c"]
+    nxt = {rid: 5 + i for i, rid in enumerate(live)}
+    used = 0
+    for step in range(30):
+        if step == 6:     # a request ends
+            for r in (eager, graph):
+                r.cache.release("b")
+            live.remove("b")
+        if step == 11:    # another joins (a step of another kind in between)
+            admit("d", 15, 4)
+            live.append("d")
+            nxt["d"] = 9
+        if step == 17:    # the same requests in another order
+            live = live[::-1]
+        if step == 22:    # one of them is served alone for a step
+            l = both([StepEntry("a", [nxt["a"]], [0])])
+            nxt["a"] = int(torch.argmax(l[0]))
+        prepared = graph._prepared is not None
+        l = both([StepEntry(rid, [nxt[rid]], [0]) for rid in live])
+        used += prepared and graph._prepared is not None
+        nxt.update({rid: int(torch.argmax(l[i])) for i, rid in enumerate(live)})
+    assert used > 10      # the prepared path did run in the quiet stretches
+    for r in (eager, graph):
+        for rid in live:
+            r.cache.release(rid)
+        r.cache.check()
+        assert r.cache.free_pages() == 48
+
+
 def test_graph_with_many_requests_replays_like_eager(models):
     """More than 16 decoded tokens a step: the projections go to the vendor library inside the
     captured graph; replays must still equal eager steps, several times over."""
