@@ -386,7 +386,10 @@ def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple
     cus = _NUM_CUS.get(device)
     if cus is None:
         cus = _NUM_CUS[device] = torch.cuda.get_device_properties(device).multi_processor_count
-    wanted = max(1, min(-(-4 * cus // max(pairs, 1)), ATT_MAX_CHUNKS, -(-bound // ATT_STEP)))
+    # the shortest chunk: one step of 128 keys while that still leaves compute units idle, else two
+    # (measured at 4096 keys: one token 12.7 against 13.4 us, eight tokens 16.9 against 15.0 us)
+    min_span = ATT_STEP if pairs * -(-bound // ATT_STEP) <= cus else 2 * ATT_STEP
+    wanted = max(1, min(-(-4 * cus // max(pairs, 1)), ATT_MAX_CHUNKS, -(-bound // min_span)))
     span = -(-bound // (wanted * ATT_STEP)) * ATT_STEP
     return span, -(-max_total_len // span)
 
