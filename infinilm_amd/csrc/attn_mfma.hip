@@ -298,7 +298,7 @@ __global__ void __launch_bounds__(256, 2)
 attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ kc,
                  const bf16* __restrict__ vc, const int* __restrict__ block_tables, const int* __restrict__ seg,
                  const int* __restrict__ pos, const int* __restrict__ tiles, int nh, int nkv, int page,
-                 int max_blocks, int q_stride, int out_stride, float scale_log2e, int window) {
+                 int max_blocks, int q_stride, int out_stride, float scale_log2e, int window, int pair_base) {
     constexpr int D = D16 * 16;
     constexpr int KS = (D + 31) / 32;
     constexpr int KROW = D + 8;         // padded rows: conflict-free 16-byte reads of 16 rows
@@ -306,9 +306,16 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     __shared__ __attribute__((aligned(16))) bf16 Ks[ATT_TK][KROW];
     __shared__ __attribute__((aligned(16))) bf16 Vs[D][VROW];
     __shared__ int bt_s[ATT_BT_LDS];
-    // the longest tiles (latest positions) are dispatched first
-    const int tile_id = gridDim.x - 1 - blockIdx.x;
-    const int by = blockIdx.y;
+    // Items (tile, head group) in descending order of length: the longest tiles (latest positions)
+    // are dispatched first.  When the whole launch is resident at once (at most two workgroups a
+    // compute unit), workgroups w and w + pair_base land on the same unit (workgroups go to the
+    // eight dies in turn and to a die's units in turn): the second of them then takes the items
+    // from the short end, so that every unit holds a long and a short one.
+    const int n_items = gridDim.x * gridDim.y;
+    const int w = blockIdx.y * gridDim.x + blockIdx.x;
+    const int item = (pair_base > 0 && w >= pair_base) ? n_items - 1 - (w - pair_base) : w;
+    const int tile_id = gridDim.x - 1 - item / gridDim.y;
+    const int by = item % gridDim.y;
     const int t0 = tiles[2 * tile_id], ntok = tiles[2 * tile_id + 1];
     const int G = nh / nkv;
     const int HG = (G + 15) / 16;
@@ -747,6 +754,17 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
 
 extern "C" int ilm_attn_tile_tokens() { return ATT_TT; }
 
+static int att_num_cus() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
 extern "C" int ilm_attn_tile(void* out, const void* q, const void* kc, const void* vc, const void* block_tables,
                              const void* seg, const void* pos, const void* tiles, int n_tiles, int nh, int nkv,
                              int d, int page, int max_blocks, int q_stride, int out_stride, float scale,
@@ -760,8 +778,11 @@ extern "C" int ilm_attn_tile(void* out, const void* q, const void* kc, const voi
     ILM_REQUIRE(nkv * HG <= 65535, "attn_tile: grid too large");
     dim3 grid(n_tiles, nkv * HG);
     const float sl2 = scale * 1.4426950408889634f;
+    const int cus = att_num_cus();
+    const long long n_items = (long long)n_tiles * nkv * HG;
+    const int pair_base = (n_items > cus && n_items <= 2 * cus) ? cus : 0;
 #define AT_ARGS (bf16*)out, (const bf16*)q, (const bf16*)kc, (const bf16*)vc, (const int*)block_tables, (const int*)seg, \
-                (const int*)pos, (const int*)tiles, nh, nkv, page, max_blocks, q_stride, out_stride, sl2, window
+                (const int*)pos, (const int*)tiles, nh, nkv, page, max_blocks, q_stride, out_stride, sl2, window, pair_base
 #define AT_CASE(D16)                                                                   \
     case D16:                                                                          \
         if (page % ATT_TK == 0) attn_tile_kernel<D16, true><<<grid, 256, 0, stream>>>(AT_ARGS);  \
