@@ -77,7 +77,8 @@ class LLMEngine:
         done = self.scheduler.update(out, sampled)
         c = self.counters
         c["steps"] += 1
-        c["prompt_tokens"] += sum(e.num_tokens for e in out.entries if e.start < e.request.get_prompt_length())
+        if len(tokens) != len(out.entries) or out.entries[0].num_tokens != 1:   # not a step of decoded tokens alone
+            c["prompt_tokens"] += sum(e.num_tokens for e in out.entries if e.start < e.request.get_prompt_length())
         c["generated_tokens"] += len(tokens)
         c["step_s"] += t2 - t1
         c["sample_s"] += t3 - t2

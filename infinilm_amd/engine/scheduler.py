@@ -134,7 +134,33 @@ class Scheduler:
         self.waiting.appendleft(victim)
         out.preempted.append(victim)
 
+    def _steady_decode(self) -> Optional[SchedulerOutput]:
+        """The plan of a step in which every running request decodes one token and nothing else can
+        happen (nobody can be admitted, and the pools hold a page for each request in case it starts
+        one): the same plan as the full procedure gives, without its page arithmetic."""
+        running = self.running
+        R = len(running)
+        if R == 0 or R > self.max_num_batched_tokens or (self.waiting and R < self.max_num_seqs):
+            return None
+        for g in self.cache.groups:
+            if g.pool.num_free < R:
+                return None
+        out = SchedulerOutput()
+        entries = out.entries
+        for req in running:            # `running` is in order of admission
+            start = req.num_computed_tokens
+            if req.num_known_tokens() - start != 1 or not req.output_token_ids:
+                return None
+            entries.append(ScheduledEntry(req, start, 1, True))
+        self.log.append({"decode": R, "portions": [], "preempted": 0,
+                         "free_pages": [g.pool.num_free for g in self.cache.groups]})
+        return out
+
     def schedule(self) -> SchedulerOutput:
+        steady = self._steady_decode()
+        return steady if steady is not None else self._schedule_in_full()
+
+    def _schedule_in_full(self) -> SchedulerOutput:
         out = SchedulerOutput()
         promised = [0] * len(self.cache.groups)
         budget = self.max_num_batched_tokens
@@ -215,7 +241,7 @@ class Scheduler:
                 self._fail(victim, "no_capacity: the request cannot make progress with the whole pool to itself")
             else:
                 self._preempt(victim, out)
-                return self._merge(out, self.schedule())
+                return self._merge(out, self._schedule_in_full())
         self.log.append({"decode": sum(1 for e in out.entries if e.num_tokens == 1 and e.start > 0),
                          "portions": [e.num_tokens for e in out.entries if not (e.num_tokens == 1 and e.start > 0)],
                          "preempted": len(out.preempted), "free_pages": [g.pool.num_free for g in self.cache.groups]})

@@ -278,7 +278,7 @@ class StepRunner:
         With `enable_graph`, a step of single decoded tokens that wants each token's logits replays
         a captured HIP graph; the returned tensor is then the graph's output buffer, valid until
         the next such step."""
-        if self.enable_graph and taps is None and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+        if self.enable_graph and taps is None and all(len(e.tokens) == 1 and len(e.want) == 1 and e.want[0] == 0 for e in entries):
             key = self._graph_key(entries)
             if key not in self._graphs:
                 self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
@@ -334,10 +334,11 @@ class StepRunner:
                 # built while the device ran the last step: only the token ids are new
                 dev, host, turn, tok_off = prep[2]
                 V = self.model.spec.vocab_size
-                for i, e in enumerate(entries):
-                    if not 0 <= e.tokens[0] < V:
-                        raise ValueError(f"request {e.req_id!r}: token id {e.tokens[0]} is outside the vocabulary of {V}")
-                    host[tok_off + i] = e.tokens[0]
+                toks = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=R)
+                if toks.min() < 0 or toks.max() >= V:
+                    bad = next(e for e in entries if not 0 <= e.tokens[0] < V)
+                    raise ValueError(f"request {bad.req_id!r}: token id {bad.tokens[0]} is outside the vocabulary of {V}")
+                host.numpy()[tok_off:tok_off + R] = toks
                 self._copy_to_device(dev, host, turn)
             else:
                 fresh = self.build_batch(entries, min_blocks=width, device_buffer=buf)

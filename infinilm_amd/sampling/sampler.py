@@ -11,6 +11,7 @@ from __future__ import annotations
 
 from typing import List, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from .. import kernels
@@ -36,6 +37,7 @@ def uniform_for(seed: int, request_key: int, index: int) -> float:
 class Sampler:
     def __init__(self, seed: int = 0):
         self.seed = int(seed)
+        self._staging = None    # pinned host memory for the rows' parameters
 
     def sample(self, logits: torch.Tensor, rows: Sequence[Tuple[SamplingParams, int, int]]) -> List[int]:
         """`rows[i]` = (params, request key, index of the token being generated) for logits[i]."""
@@ -46,10 +48,19 @@ class Sampler:
             return []
         if all(p.greedy for p, _, _ in rows):
             return kernels.argmax(logits).tolist()
+        # temperature, top_k, top_p and the uniform numbers in one pinned buffer and one copy that
+        # queues behind the step (a copy from pageable memory would make the host wait for the step
+        # and the device wait for four copies)
         dev = logits.device
-        temp = torch.tensor([p.temperature for p, _, _ in rows], dtype=torch.float32).to(dev)
-        top_k = torch.tensor([p.top_k for p, _, _ in rows], dtype=torch.int32).to(dev)
-        top_p = torch.tensor([p.top_p for p, _, _ in rows], dtype=torch.float32).to(dev)
-        u = torch.tensor([uniform_for(self.seed if p.seed is None else p.seed, key, idx) for p, key, idx in rows],
-                         dtype=torch.float32).to(dev)
-        return kernels.sample(logits, temp, top_k, top_p, u).tolist()
+        if self._staging is None or self._staging.numel() < 4 * n:
+            self._staging = torch.empty((4 * max(n, 64),), dtype=torch.float32, pin_memory=dev.type == "cuda")
+        host = self._staging[:4 * n]
+        h = host.numpy()
+        h[0:n] = [p.temperature for p, _, _ in rows]
+        h[n:2 * n].view(np.int32)[:] = [p.top_k for p, _, _ in rows]
+        h[2 * n:3 * n] = [p.top_p for p, _, _ in rows]
+        h[3 * n:4 * n] = [uniform_for(self.seed if p.seed is None else p.seed, key, idx) for p, key, idx in rows]
+        d = torch.empty((4 * n,), dtype=torch.float32, device=dev)
+        d.copy_(host, non_blocking=True)
+        tokens = kernels.sample(logits, d[0:n], d[n:2 * n].view(torch.int32), d[2 * n:3 * n], d[3 * n:4 * n])
+        return tokens.tolist()   # waits for the stream: the staging buffer is free again after this

@@ -286,6 +286,7 @@ def test_every_admitted_request_finishes_under_random_load(seed):
                   policy=rng.choice(["optimistic", "reserve_full"]), max_positions=1000)
     reqs = [_req(f"r{i}", rng.randint(1, 25), max_tokens=rng.randint(1, 12)) for i in range(12)]
     pending = list(reqs)
+    short_plans = 0
     for _ in range(2000):
         while pending and rng.random() < 0.5:
             s.add_request(pending.pop(0))
@@ -293,6 +294,12 @@ def test_every_admitted_request_finishes_under_random_load(seed):
             if not pending:
                 break
             continue
+        steady = s._steady_decode()
+        if steady is not None:   # the short way for steps of decoded tokens alone plans what the full procedure plans
+            full = s._schedule_in_full()
+            key = lambda o: [(e.request.request_id, e.start, e.num_tokens, e.samples) for e in o.entries]
+            assert key(steady) == key(full) and not full.preempted and s.log[-1] == s.log[-2]
+            short_plans += 1
         out = s.schedule()
         assert len({e.request.request_id for e in out.entries}) == len(out.entries) <= 3
         assert out.num_tokens <= s.max_num_batched_tokens
@@ -300,6 +307,7 @@ def test_every_admitted_request_finishes_under_random_load(seed):
             c.reserve(e.request.request_id, e.num_tokens); c.commit(e.request.request_id, e.num_tokens)
         s.update(out, {e.request.request_id: 7 for e in out.entries if e.samples})
         c.check()
+    assert short_plans > 0
     assert all(r.is_finished() for r in reqs)
     ok = [r for r in reqs if r.status == RequestStatus.FINISHED]
     assert all(r.get_num_generated_tokens() == r.sampling_params.max_tokens for r in ok)
