@@ -9,7 +9,7 @@
 // Two kernels:
 //  * stream:  RT tiles of 16 W rows per workgroup, up to 4 token groups; the X fragments are
 //             re-read from L2 for every workgroup.  Any K (multiple of 8), any M <= 64.
-//  * resident (M <= 16, K <= 16 waves * KSTEPS * 32): each wave keeps the X fragments of its
+//  * resident (M <= 16 and K <= 8192, or M <= 32 and K <= 4096): each wave keeps the X fragments of its
 //             K slice in registers and the workgroup walks over W row tiles, prefetching the next
 //             tile's rows while the current one is reduced; X is read once per workgroup.
 // K must be a multiple of 8 (16-byte loads); rows of X and W must be 16-byte aligned.
@@ -120,29 +120,36 @@ gemm_skinny_stream_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const 
     }
 }
 
-// M <= 16.  WAVES waves of KSTEPS k-steps (32 elements each) cover K; X fragments stay in registers.
-template <int WAVES, int KSTEPS, typename TC>
+// M <= 16 MG.  WAVES waves of KSTEPS k-steps (32 elements each) cover K; the X fragments of MG groups
+// of 16 rows stay in registers, so a W fragment read once serves MG matrix instructions.
+template <int WAVES, int KSTEPS, int MG, typename TC>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_resident_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
                             const bf16* __restrict__ bias, int M, int N, int K, int lda, int ldw, int ldc,
                             float alpha, int ntiles) {
-    __shared__ float part[2][WAVES][64][4];
+    static_assert(WAVES * 64 >= 256 * MG, "one reducing thread an output");
+    __shared__ float part[2][MG][WAVES][64][4];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, q = lane >> 4;
     const int s0 = wave * KSTEPS;
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     const int k8_last = (K >> 3) - 1;
-    uint4 xf[KSTEPS];
+    uint4 xf[MG][KSTEPS];
     int k8c[KSTEPS];
-    {
-        const uint4* xp = reinterpret_cast<const uint4*>(X + (size_t)(r < M ? r : 0) * lda);
+#pragma unroll
+    for (int u = 0; u < KSTEPS; ++u) {
+        const int k8 = (s0 + u) * 4 + q;
+        k8c[u] = k8 < k8_last ? k8 : k8_last;
+    }
+#pragma unroll
+    for (int g = 0; g < MG; ++g) {
+        const int row = g * 16 + r;
+        const uint4* xp = reinterpret_cast<const uint4*>(X + (size_t)(row < M ? row : 0) * lda);
 #pragma unroll
         for (int u = 0; u < KSTEPS; ++u) {
-            const int k8 = (s0 + u) * 4 + q;
-            k8c[u] = k8 < k8_last ? k8 : k8_last;
             const uint4 v = xp[k8c[u]];
             // zero fragments beyond K or beyond M make the clamped W loads harmless
-            xf[u] = (k8 <= k8_last && r < M) ? v : zero;
+            xf[g][u] = ((s0 + u) * 4 + q <= k8_last && row < M) ? v : zero;
         }
     }
     uint4 a[KSTEPS];
@@ -155,9 +162,13 @@ gemm_skinny_resident_kernel(TC* __restrict__ C, const bf16* __restrict__ X, cons
     }
     int buf = 0;
     for (; tile < ntiles; tile += gridDim.x) {
-        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+        f32x4 acc[MG];
 #pragma unroll
-        for (int u = 0; u < KSTEPS; ++u) acc = mfma16(a[u], xf[u], acc);
+        for (int g = 0; g < MG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u)
+#pragma unroll
+            for (int g = 0; g < MG; ++g) acc[g] = mfma16(a[u], xf[g][u], acc[g]);
         // the next tile's rows are on their way while this one is reduced
         const int next = tile + gridDim.x;
         __builtin_amdgcn_sched_barrier(0);
@@ -168,21 +179,111 @@ gemm_skinny_resident_kernel(TC* __restrict__ C, const bf16* __restrict__ X, cons
             for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
         }
         __builtin_amdgcn_sched_barrier(0);
-        *reinterpret_cast<f32x4*>(&part[buf][wave][lane][0]) = acc;
+#pragma unroll
+        for (int g = 0; g < MG; ++g) *reinterpret_cast<f32x4*>(&part[buf][g][wave][lane][0]) = acc[g];
         __syncthreads();
-        if (threadIdx.x < 256) {
-            const int e = threadIdx.x & 3, l = threadIdx.x >> 2;
+        if (threadIdx.x < 256 * MG) {
+            const int g = threadIdx.x >> 8, t = threadIdx.x & 255;
+            const int e = t & 3, l = t >> 2;
             float v = 0.f;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) v += part[buf][w][l][e];
+            for (int w = 0; w < WAVES; ++w) v += part[buf][g][w][l][e];
             const int n = tile * 16 + (l >> 4) * 4 + e;
-            const int m = l & 15;
+            const int m = g * 16 + (l & 15);
             if (n < N && m < M) {
                 if (bias != nullptr) v += to_f32(bias[n]);
                 C[(size_t)m * ldc + n] = from_f32<TC>(alpha * v);
             }
         }
         buf ^= 1;  // the other buffer is free: its readers passed the barrier above one tile ago
+    }
+}
+
+// The fused gate/up projection of a feed-forward with the SwiGLU in its epilogue (few rows of X):
+// W holds the gate rows [0, I) and the up rows [I, 2I).  A workgroup multiplies the gate tile and
+// the up tile of the same 16 outputs one after the other; the thread that reduces output (m, n) of
+// the first also reduces (m, n) of the second and stores act[m, n] = silu(gate) * up.  The
+// intermediate [M, 2I] never goes to memory and the following projection reads plain rows.
+// Gate and up are rounded to bfloat16 before the activation, as the unfused path stores them.
+template <int WAVES, int KSTEPS, int MG>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_gateup_swiglu_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
+                          const bf16* __restrict__ bias, int M, int I, int K, int lda, int ldw, int ldc, int ntiles) {
+    static_assert(WAVES * 64 >= 256 * MG, "one reducing thread an output");
+    __shared__ float part[2][MG][WAVES][64][4];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = lane & 15, q = lane >> 4;
+    const int s0 = wave * KSTEPS;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    const int k8_last = (K >> 3) - 1;
+    uint4 xf[MG][KSTEPS];
+    int k8c[KSTEPS];
+#pragma unroll
+    for (int u = 0; u < KSTEPS; ++u) {
+        const int k8 = (s0 + u) * 4 + q;
+        k8c[u] = k8 < k8_last ? k8 : k8_last;
+    }
+#pragma unroll
+    for (int g = 0; g < MG; ++g) {
+        const int row = g * 16 + r;
+        const uint4* xp = reinterpret_cast<const uint4*>(X + (size_t)(row < M ? row : 0) * lda);
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u) {
+            const uint4 v = xp[k8c[u]];
+            xf[g][u] = ((s0 + u) * 4 + q <= k8_last && row < M) ? v : zero;
+        }
+    }
+    // this lane's W row of a tile's gate half (0) or up half (1)
+    auto w_row = [&](int t, int hf) -> const uint4* {
+        const int n = (t * 16 + r < I) ? t * 16 + r : I - 1;
+        return reinterpret_cast<const uint4*>(W + (size_t)(n + hf * I) * ldw);
+    };
+    uint4 a[KSTEPS];
+    int tile = blockIdx.x;
+    if (tile < ntiles) {
+        const uint4* wp = w_row(tile, 0);
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
+    }
+    const int et = threadIdx.x < 256 * MG ? threadIdx.x : 0;
+    const int eg = et >> 8, e = et & 3, l = (et & 255) >> 2;
+    const int m = eg * 16 + (l & 15);
+    int buf = 0;
+    for (; tile < ntiles; tile += gridDim.x) {
+        const int n = tile * 16 + (l >> 4) * 4 + e;
+        const bool writer = threadIdx.x < 256 * MG && n < I && m < M;
+        float val[2];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            f32x4 acc[MG];
+#pragma unroll
+            for (int g = 0; g < MG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < KSTEPS; ++u)
+#pragma unroll
+                for (int g = 0; g < MG; ++g) acc[g] = mfma16(a[u], xf[g][u], acc[g]);
+            // the next tile's rows are on their way while this one is reduced
+            const int nt = hf == 0 ? tile : tile + gridDim.x;
+            __builtin_amdgcn_sched_barrier(0);
+            if (nt < ntiles) {
+                const uint4* wp = w_row(nt, hf == 0 ? 1 : 0);
+#pragma unroll
+                for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < MG; ++g) *reinterpret_cast<f32x4*>(&part[buf][g][wave][lane][0]) = acc[g];
+            __syncthreads();
+            float v = 0.f;
+            if (threadIdx.x < 256 * MG) {
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) v += part[buf][eg][w][l][e];
+                if (bias != nullptr && writer) v += to_f32(bias[n + hf * I]);
+            }
+            val[hf] = to_f32(from_f32<bf16>(v));
+            buf ^= 1;  // the other buffer is free: its readers passed the barrier above one tile ago
+        }
+        if (writer) C[(size_t)m * ldc + n] = from_f32<bf16>(val[0] / (1.0f + expf(-val[0])) * val[1]);
     }
 }
 
@@ -211,17 +312,18 @@ extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void
     ILM_REQUIRE(out_dtype == ILM_DTYPE_BF16 || out_dtype == ILM_DTYPE_F32, "gemm_skinny: unknown output dtype %d", out_dtype);
     const int mg = (M + 15) / 16;
     const int ksteps = (K + 31) / 32;
-    const bool can_resident = M <= 16 && ksteps <= 16 * 16;
-    // measured on MI355X at the 8B shapes: resident wins for M <= 16 where it applies, the 16-wave
-    // stream shape for long K, two row tiles when X has more than 16 rows and W is tall
+    // two groups of 16 rows take the 8-wave shapes (256 registers a wave): K up to 8 * 16 k-steps
+    const bool can_resident = (M <= 16 && ksteps <= 16 * 16) || (M <= 32 && ksteps <= 8 * 16);
+    // measured on MI355X at the 8B shapes: resident wins where it applies, the 16-wave stream shape
+    // for long K, two row tiles when X has more than 32 rows and W is tall
     if (variant == 0) variant = can_resident ? 4 : (M <= 16 ? 3 : (N >= 8192 ? 2 : 1));
     if (variant == 4) {
-        ILM_REQUIRE(can_resident, "gemm_skinny: the resident kernel needs M <= 16 and K <= 8192");
+        ILM_REQUIRE(can_resident, "gemm_skinny: the resident kernel needs M <= 16 and K <= 8192, or M <= 32 and K <= 4096");
         const int ntiles = (N + 15) / 16;
-#define SR_CASE(WV, KS, TC)                                                                                 \
+#define SR_CASE(WV, KS, MGR, PER_CU, TC)                                                                    \
     {                                                                                                       \
-        const int grid = ntiles < num_cus() * (WV == 16 ? 1 : 2) ? ntiles : num_cus() * (WV == 16 ? 1 : 2); \
-        gemm_skinny_resident_kernel<WV, KS, TC><<<grid, WV * 64, 0, stream>>>(                              \
+        const int grid = ntiles < num_cus() * PER_CU ? ntiles : num_cus() * PER_CU;                         \
+        gemm_skinny_resident_kernel<WV, KS, MGR, TC><<<grid, WV * 64, 0, stream>>>(                         \
             (TC*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha, ntiles); \
     }
         // measured on MI355X at K = 4096: 8 waves of 16 k-steps (more loads in flight a wave) win where the
@@ -231,12 +333,17 @@ extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void
         static int fat = -1;
         if (fat < 0) { const char* e = getenv("INFINILM_AMD_SKINNY_FAT"); fat = e ? atoi(e) : 1; }
         const bool fat_waves = fat && ksteps > 8 * 8 && ksteps <= 8 * 16 && (ntiles <= num_cus() || ntiles >= 4 * num_cus());
-#define SR_DISPATCH(TC)                                   \
-    if (ksteps <= 8 * 4) SR_CASE(8, 4, TC)                \
-    else if (ksteps <= 8 * 8) SR_CASE(8, 8, TC)           \
-    else if (fat_waves) SR_CASE(8, 16, TC)                \
-    else if (ksteps <= 16 * 8) SR_CASE(16, 8, TC)         \
-    else SR_CASE(16, 16, TC)
+#define SR_DISPATCH(TC)                                         \
+    if (mg == 2) {                                              \
+        if (ksteps <= 8 * 4) SR_CASE(8, 4, 2, 2, TC)            \
+        else if (ksteps <= 8 * 8) SR_CASE(8, 8, 2, 2, TC)       \
+        else SR_CASE(8, 16, 2, 1, TC)                           \
+    }                                                           \
+    else if (ksteps <= 8 * 4) SR_CASE(8, 4, 1, 2, TC)           \
+    else if (ksteps <= 8 * 8) SR_CASE(8, 8, 1, 2, TC)           \
+    else if (fat_waves) SR_CASE(8, 16, 1, 2, TC)                \
+    else if (ksteps <= 16 * 8) SR_CASE(16, 8, 1, 1, TC)         \
+    else SR_CASE(16, 16, 1, 1, TC)
         if (out_dtype == ILM_DTYPE_BF16) { SR_DISPATCH(bf16) } else { SR_DISPATCH(float) }
 #undef SR_DISPATCH
 #undef SR_CASE
@@ -274,5 +381,35 @@ extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void
 #undef SK_MG
 #undef SK_CASE
     ILM_LAUNCH_CHECK("gemm_skinny_stream");
+    return 0;
+}
+
+// act [M, ldc] = silu(X Wg^T + bg) * (X Wu^T + bu) with W = [Wg; Wu] of 2 I rows (bias of 2 I entries or null).
+extern "C" int ilm_gemm_gateup_swiglu(void* C, int ldc, const void* X, int lda, const void* W, int ldw, const void* bias,
+                                      int M, int I, int K, hipStream_t stream) {
+    ILM_REQUIRE(M > 0 && M <= 32 && I > 0 && K > 0, "gemm_gateup_swiglu: needs 1 <= M <= 32, got M=%d I=%d K=%d", M, I, K);
+    ILM_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldc >= I,
+                "gemm_gateup_swiglu: K=%d lda=%d ldw=%d ldc=%d", K, lda, ldw, ldc);
+    ILM_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_gateup_swiglu: operands must be 16-byte aligned");
+    const int ksteps = (K + 31) / 32;
+    ILM_REQUIRE(ksteps <= (M <= 16 ? 16 * 16 : 8 * 16), "gemm_gateup_swiglu: K=%d is beyond %d", K, M <= 16 ? 8192 : 4096);
+    const int ntiles = (I + 15) / 16;
+#define GU_CASE(WV, KS, MGR, PER_CU)                                                                        \
+    {                                                                                                       \
+        const int grid = ntiles < num_cus() * PER_CU ? ntiles : num_cus() * PER_CU;                         \
+        gemm_gateup_swiglu_kernel<WV, KS, MGR><<<grid, WV * 64, 0, stream>>>(                               \
+            (bf16*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, I, K, lda, ldw, ldc, ntiles);   \
+    }
+    if (M > 16) {
+        if (ksteps <= 8 * 4) GU_CASE(8, 4, 2, 2)
+        else if (ksteps <= 8 * 8) GU_CASE(8, 8, 2, 2)
+        else GU_CASE(8, 16, 2, 1)
+    }
+    else if (ksteps <= 8 * 4) GU_CASE(8, 4, 1, 2)
+    else if (ksteps <= 8 * 8) GU_CASE(8, 8, 1, 2)
+    else if (ksteps <= 8 * 16) GU_CASE(8, 16, 1, 2)
+    else GU_CASE(16, 16, 1, 1)
+#undef GU_CASE
+    ILM_LAUNCH_CHECK("gemm_gateup_swiglu");
     return 0;
 }

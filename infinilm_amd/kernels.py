@@ -205,10 +205,10 @@ def qkv_rope_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
                   slots: Optional[torch.Tensor], nh: int, nkv: int, d: int, rd: int) -> Optional[torch.Tensor]:
     """The fused projection x w^T (+ bias) of a few rows, q and k rotated and k, v written to the cache
     in the product's epilogue.  Returns the rotated q [T, nh*d], or None where the fused kernel does
-    not apply (more than 16 rows, float32, a partly rotated or odd-sized head): the caller then
+    not apply (more than 32 rows, float32, a partly rotated or odd-sized head): the caller then
     runs the projection and `rope_kvwrite` one after the other."""
     M, K = x.shape
-    if not (USE_QKV_ROPE and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and M <= 16 and rd == d and d % 32 == 0
+    if not (USE_QKV_ROPE and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and _few_rows(M, K) and rd == d and d % 32 == 0
             and K % 8 == 0 and K <= 8192 and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
             and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         return None
@@ -257,6 +257,12 @@ def gather_rows(x: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
 
 _LIBRARY_F32_OUT = [True]   # cleared when torch.mm refuses out_dtype
 KSPLIT_SPAN = 4096  # K range of one part of the K-split few-rows product (ilm_gemm_ksplit_max_k(1))
+# Rows up to which the products keep X in registers (16 or 32; 32 only for K up to 4096 a workgroup)
+FEW_ROWS = int(os.environ.get("INFINILM_AMD_FEW_ROWS", "32"))
+
+
+def _few_rows(M: int, K: int) -> bool:
+    return M <= 16 or (M <= FEW_ROWS and K <= 4096)
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, alpha: float = 1.0,
@@ -288,20 +294,22 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     # projection 22 -> 17 and 25 -> 19; up to 64 rows the library and a one-part sum are as fast)
     if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS:
         return _gemm_mid(a, w, K, False)
-    if fast and aligned and plain and allow_parts and out is None and M <= 16 and K > 2 * KSPLIT_SPAN and USE_KSPLIT:
+    if fast and aligned and plain and allow_parts and out is None and M <= max(16, FEW_ROWS) and K > 2 * KSPLIT_SPAN and USE_KSPLIT:
         kb = -(-K // KSPLIT_SPAN)
         parts = torch.empty((kb, M, N), dtype=F32, device=a.device)
         _run("ilm_gemm_ksplit", parts.data_ptr(), _DT[F32], N, M * N, kb, w.data_ptr(), w.stride(0), None, 1.0,
              M, N, K, a.data_ptr(), a.stride(0), 0, _stream())
         return parts
-    if fast and aligned and allow_parts and out is None and M <= 16:
+    few = fast and aligned and _few_rows(M, K)
+    if few and allow_parts and out is None:
         out_dtype = F32   # a branch on its way into the float32 residual sum need not be rounded first
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     library_ok = fast and plain and out_dtype == BF16 and USE_LIBRARY_GEMM
-    # measured at the 8B shapes: the few-rows kernel beats the vendor library up to 16 rows and loses
-    # to it above (its X fragments are re-read from L2 for every 16 rows of W)
-    if (M > 16 and fast and bias is None and out_dtype == F32 and USE_LIBRARY_GEMM and _LIBRARY_F32_OUT[0]
+    # measured at the 8B shapes: the few-rows kernel with X in registers beats the vendor library (up to
+    # 32 rows: gate_up 53 against 62 us, o projection 14 against 18); where X no longer fits the
+    # registers it loses (its X fragments are re-read from L2 for every 16 rows of W)
+    if (not few and M > 16 and fast and bias is None and out_dtype == F32 and USE_LIBRARY_GEMM and _LIBRARY_F32_OUT[0]
             and M <= 65535):
         # bfloat16 operands, float32 accumulation and result (the output head with many rows)
         try:
@@ -315,7 +323,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
             if alpha != 1.0:
                 _run("ilm_scale_rows", out.data_ptr(), M, N, out.stride(0), float(alpha), _stream())
             return out
-    if fast and aligned and M <= 64 and not (M > 16 and library_ok):
+    if fast and aligned and M <= 64 and (few or not library_ok):
         _run("ilm_gemm_skinny", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
              w.stride(0), out.stride(0), float(alpha), _DT[out_dtype], SKINNY_VARIANT, _stream())
         return out
@@ -348,15 +356,38 @@ def _gemm_mid(x: torch.Tensor, w: torch.Tensor, K: int, act: bool) -> torch.Tens
     return parts
 
 
+USE_GATEUP_SWIGLU = os.environ.get("INFINILM_AMD_GATEUP_SWIGLU", "1") == "1"
+
+
+def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """silu(x Wg^T + bg) * (x Wu^T + bu) for few rows in bfloat16, W = [Wg; Wu]: the fused gate/up
+    projection with the SwiGLU in its epilogue, [M, I].  None where the kernel does not apply (too many
+    rows, float32, K beyond the registers): the caller then runs the projection and the activation."""
+    M, K = x.shape
+    if not (USE_GATEUP_SWIGLU and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and x.is_cuda
+            and _few_rows(M, K) and K <= 8192 and K % 8 == 0 and w.shape[0] % 2 == 0 and w.shape[1] == K
+            and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        return None
+    _dev(x, w, bias)
+    I = w.shape[0] // 2
+    if bias is not None and (bias.shape != (2 * I,) or bias.dtype != BF16 or not bias.is_contiguous()):
+        raise KernelError("bias does not fit the fused gate/up projection")
+    out = torch.empty((M, I), dtype=BF16, device=x.device)
+    _run("ilm_gemm_gateup_swiglu", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
+         _ptr(bias), M, I, K, _stream())
+    return out
+
+
 def swiglu_gemm(gate_up: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
-    """(silu(gate) * up) w^T for at most 16 rows [gate | up] in bfloat16, in one kernel: float32 parts
+    """(silu(gate) * up) w^T for at most 32 rows [gate | up] in bfloat16, in one kernel: float32 parts
     [P, M, N] for add_rmsnorm.  None when the shapes do not fit (the caller then runs the two kernels)."""
     M, two_k = gate_up.shape
     K = two_k // 2
     N = w.shape[0]
-    # (above 16 rows the activation would be recomputed by every workgroup along N: the separate kernel
+    # (above 32 rows the activation would be recomputed by every workgroup along N: the separate kernel
     # and the medium-rows product are faster, 38 against 42 us at 64 rows)
-    ok = (gate_up.dtype == BF16 and w.dtype == BF16 and not FORCE_BASIC and USE_KSPLIT and M <= 16
+    ok = (gate_up.dtype == BF16 and w.dtype == BF16 and not FORCE_BASIC and USE_KSPLIT and M <= max(16, FEW_ROWS)
           and two_k % 2 == 0
           and w.shape[1] == K and K % 8 == 0 and gate_up.stride(1) == 1 and w.stride(1) == 1 and gate_up.stride(0) % 8 == 0
           and w.stride(0) % 8 == 0 and gate_up.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and gate_up.is_cuda)

@@ -28,6 +28,9 @@ class SwiGLU(FeedForward):
         return out
 
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
+        act = kernels.gateup_swiglu_gemm(x, self.gate_up.weight, self.gate_up.bias)   # few rows: activation in the epilogue
+        if act is not None:
+            return self.down.forward(act, allow_parts=True)
         gu = self.gate_up.forward(x)
         if self.down.bias is None:
             fused = kernels.swiglu_gemm(gu, self.down.weight)   # few rows: activation inside the product

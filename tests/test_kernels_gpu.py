@@ -113,7 +113,9 @@ def test_rope_and_cache_write(K, dtype, nh, nkv, d, rd, page):
 
 @pytest.mark.parametrize("M,nh,nkv,d,Kd,page,bias", [(5, 4, 2, 32, 96, 8, False), (16, 32, 2, 128, 4096, 64, False),
                                                      (1, 3, 3, 64, 200, 16, True), (8, 16, 2, 64, 1024, 16, False),
-                                                     (3, 2, 1, 96, 8192, 4, True)])
+                                                     (3, 2, 1, 96, 8192, 4, True), (17, 4, 2, 32, 96, 8, True),
+                                                     (32, 32, 2, 128, 4096, 64, False), (24, 16, 2, 64, 1024, 16, False),
+                                                     (29, 3, 3, 96, 2056, 16, True)])
 def test_projection_with_rotation_and_cache_write_in_one_kernel(K, M, nh, nkv, d, Kd, page, bias):
     """The decode-side fused kernel against the plain product + rotation, and against the
     product kernel followed by the rotation kernel."""
@@ -188,6 +190,8 @@ def test_gemm_float32_is_true_float32(K, M, N, K_):
     (33, 200, 96, torch.bfloat16), (64, 73448, 128, torch.float32), (48, 100, 2048, torch.bfloat16),
     (7, 50, 100, torch.bfloat16),        # K no multiple of 8: the plain kernel takes it
     (100, 176, 80, torch.bfloat16), (300, 512, 256, torch.bfloat16), (65, 40, 64, torch.float32), (40, 331, 96, torch.float32),
+    (32, 4608, 4096, torch.bfloat16), (25, 331, 4096, torch.float32), (20, 100, 1032, torch.bfloat16),   # two row groups in registers
+    (31, 50, 4104, torch.bfloat16),      # K beyond what two row groups hold: the library
 ])
 def test_gemm_bfloat16(K, M, N, K_, out_dtype):
     a, w = _rand((M, K_), 11, torch.bfloat16), _rand((N, K_), 12, torch.bfloat16)
@@ -203,22 +207,27 @@ def test_gemm_bfloat16(K, M, N, K_, out_dtype):
 
 
 @pytest.mark.parametrize("M,N,K_", [(8, 4096, 16384), (1, 50, 8200), (16, 331, 12296), (17, 4096, 4096), (64, 4096, 16384),
-                                    (48, 331, 200), (35, 50, 8200), (128, 1030, 1096), (97, 64, 72)])
+                                    (48, 331, 200), (35, 50, 8200), (128, 1030, 1096), (97, 64, 72), (32, 4096, 16384),
+                                    (20, 331, 12296), (27, 50, 8200)])
 def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
     """Few rows and long K: the product comes as float32 parts; add_rmsnorm sums them in order."""
     a, w = _rand((M, K_), 14, torch.bfloat16), _rand((N, K_), 15, torch.bfloat16, 0.05)
     parts = K.gemm(a.to(DEV), w.to(DEV), allow_parts=True)
-    if 16 < M <= 64:   # the library serves these; the kernel itself is tested all the same
+    if 32 < M <= 64:   # the library serves these; the kernel itself is tested all the same
         parts = K._gemm_mid(a.to(DEV), w.to(DEV), K_, False)
-    assert parts.dim() == 3 and parts.dtype == torch.float32 and (M > 16 or parts.shape[0] == -(-K_ // 4096))
+    if parts.dim() == 2:   # short K: one float32 result
+        assert K_ <= 8192 and M <= 32
+        parts = parts[None]
+    assert parts.dim() == 3 and parts.dtype == torch.float32
+    assert M > 32 or K_ <= 8192 or parts.shape[0] == -(-K_ // 4096)
     want = P.plain_linear(a.to(F64), w.to(F64))
     _close(parts.sum(0), want, 1e-5)
     whole = K.gemm(a.to(DEV), w.to(DEV))
     assert whole.dim() == 2 and whole.dtype == torch.bfloat16
     short = K.gemm(a[:, :256].contiguous().to(DEV), w[:, :256].contiguous().to(DEV), allow_parts=True)
     # short K: one part, not rounded to bfloat16 (more than 64 rows: the medium-rows kernel with its parts;
-    # 17 to 64: the library's bfloat16)
-    assert (short.dtype == torch.float32 and short.dim() == 2) if M <= 16 else (short.dim() == 3 if M > 64 else short.dtype == torch.bfloat16)
+    # 33 to 64: the library's bfloat16)
+    assert (short.dtype == torch.float32 and short.dim() == 2) if M <= 32 else (short.dim() == 3 if M > 64 else short.dtype == torch.bfloat16)
     _close(whole, want, 6e-3)
     r = _rand((M, N), 16, scale=2.0)
     nw = _rand((N,), 17, torch.bfloat16) + 1
@@ -230,20 +239,41 @@ def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
 
 
 @pytest.mark.parametrize("M,I,N", [(8, 16384, 4096), (3, 200, 96), (16, 4104, 50), (17, 4104, 50), (40, 8192, 1024),
-                                   (64, 16384, 4096), (33, 96, 331), (128, 1000, 70), (100, 16384, 4096)])
+                                   (64, 16384, 4096), (33, 96, 331), (128, 1000, 70), (100, 16384, 4096), (32, 16384, 4096),
+                                   (24, 200, 96)])
 def test_swiglu_inside_the_down_projection(K, M, I, N):
     gu = _rand((M, 2 * I), 18, torch.bfloat16, 1.5)
     w = _rand((N, I), 19, torch.bfloat16, 0.05)
-    if M <= 16:
+    if M <= 32:
         parts = K.swiglu_gemm(gu.to(DEV), w.to(DEV))
     else:   # the medium-rows kernel's variant with the activation on the way into LDS (not on the engine's path)
         assert K.swiglu_gemm(gu.to(DEV), w.to(DEV)) is None
         parts = K._gemm_mid(gu.to(DEV), w.to(DEV), I, True)
     assert parts is not None and parts.dtype == torch.float32 and parts.shape[1:] == (M, N)
-    if M <= 16:
+    if M <= 32:
         assert parts.shape[0] == -(-I // 4096)
     act = P.plain_swiglu(gu.to(F64)[:, :I], gu.to(F64)[:, I:])
     _close(parts.sum(0), P.plain_linear(act, w.to(F64)), 6e-3)   # the activation is rounded to bfloat16 once
+
+
+@pytest.mark.parametrize("M,I,Kd,bias", [(8, 16384, 4096, False), (3, 200, 96, True), (16, 331, 1032, False), (17, 331, 1032, True),
+                                         (32, 4096, 4096, False), (5, 50, 8192, True), (24, 96, 200, False)])
+def test_gate_up_projection_with_the_activation_in_its_epilogue(K, M, I, Kd, bias):
+    """One kernel for silu(x Wg^T) * (x Wu^T) against the plain formula and against the projection
+    followed by the activation kernel (gate and up rounded to bfloat16 at the same place)."""
+    x, w = _rand((M, Kd), 31, torch.bfloat16), _rand((2 * I, Kd), 32, torch.bfloat16, scale=2.0 * Kd ** -0.5)
+    b = _rand((2 * I,), 33, torch.bfloat16) if bias else None
+    dev = lambda t: None if t is None else t.to(DEV)
+    act = K.gateup_swiglu_gemm(dev(x), dev(w), dev(b))
+    assert act is not None and act.shape == (M, I) and act.dtype == torch.bfloat16
+    y = P.plain_linear(x.to(F64), w.to(F64), None if b is None else b.to(F64))
+    _close(act, P.plain_swiglu(y[:, :I], y[:, I:]), 1e-2)
+    two = K.swiglu(K.gemm(dev(x), dev(w), dev(b)))
+    assert (act.float() - two.float()).abs().max() <= 2 ** -6 * max(float(two.float().abs().max()), 1e-6)
+    assert K.gateup_swiglu_gemm(dev(x.float()), dev(w.float()), None) is None          # float32: not this kernel
+    if M <= 32:
+        big = _rand((33, Kd), 34, torch.bfloat16)
+        assert K.gateup_swiglu_gemm(dev(big), dev(w), dev(b)) is None                  # too many rows
 
 
 def _paged(k, v, page, n_pages, seed, dtype):
