@@ -406,10 +406,14 @@ _NUM_CUS: dict = {}
 def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple:
     """(keys a chunk, chunks) of the chunked single-token attention for `pairs` = tokens x head groups.
 
-    Enough chunks that the launch has about four workgroups a compute unit (few tokens: short
-    chunks, latency counts; many tokens: long chunks, fewer partial results to write and merge), at
-    most ATT_MAX_CHUNKS.  The length is first rounded up the way the step function rounds its graphs'
-    block tables (pages: 4, 8, 16, ...), so that an eager step and a replayed one cut alike."""
+    A chunk is a whole number of steps of ATT_STEP keys.  Few tokens: one step a chunk (latency
+    counts, the chip is not full anyway).  Up to four steps as long as the launch still has a
+    workgroup for every compute unit (fewer partial results to write and merge), and beyond that
+    while it still has two for each.  Measured at the 8B head shape, 4096 keys, kernel + merge:
+    8 tokens 17.0 us with 256 keys a chunk (128: 18.4, 512: 20.2); 16 tokens 22.4 with 512 (256:
+    24.0); 32 tokens 34.3 with 512 (256: 40.0, 1024: 36.5); 64 tokens 57.5 with 1024 (512: 60.5).
+    At most ATT_MAX_CHUNKS chunks.  The length is first rounded up the way the step function rounds
+    its graphs' block tables (pages: 4, 8, 16, ...), so that an eager step and a replayed one cut alike."""
     pages = 4
     while pages * page < max_total_len:
         pages *= 2
@@ -417,11 +421,18 @@ def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple
     cus = _NUM_CUS.get(device)
     if cus is None:
         cus = _NUM_CUS[device] = torch.cuda.get_device_properties(device).multi_processor_count
-    # the shortest chunk: one step of 128 keys while that still leaves compute units idle, else two
-    # (measured at 4096 keys: one token 12.7 against 13.4 us, eight tokens 16.9 against 15.0 us)
-    min_span = ATT_STEP if pairs * -(-bound // ATT_STEP) <= cus else 2 * ATT_STEP
-    wanted = max(1, min(-(-4 * cus // max(pairs, 1)), ATT_MAX_CHUNKS, -(-bound // min_span)))
-    span = -(-bound // (wanted * ATT_STEP)) * ATT_STEP
+    steps = -(-bound // ATT_STEP)
+    pairs = max(pairs, 1)
+    workgroups = lambda per_chunk: pairs * -(-steps // per_chunk)
+    per_chunk = 1
+    for n in (2, 3, 4):
+        if workgroups(n) >= cus:
+            per_chunk = n
+    while per_chunk >= 4 and 2 * per_chunk <= steps and workgroups(2 * per_chunk) >= 2 * cus:
+        per_chunk *= 2
+    while -(-steps // per_chunk) > ATT_MAX_CHUNKS:
+        per_chunk += 1
+    span = per_chunk * ATT_STEP
     return span, -(-max_total_len // span)
 
 
