@@ -25,16 +25,19 @@ template <int GF_WAVES, int GF_KSTEPS, int MG, bool ACT, typename TC>
 __global__ void __launch_bounds__(GF_WAVES * 64)
 gemm_ksplit_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
                    const bf16* __restrict__ bias, int M, int N, int K, int lda, int ldw, int ldc, float alpha,
-                   int ntiles, size_t c_part_stride) {
+                   int ntiles, size_t c_part_stride, int kspan, int ks) {
+    // kspan <= GF_KSPAN: K a part really covers (K spread evenly over the parts, a multiple of 32);
+    // ks <= GF_KSTEPS: k-steps a wave really takes (the part spread evenly over the waves); its other
+    // slots load its first address again (a cache hit, no branch around the loads) and multiply by zeros
     static_assert(GF_WAVES * 64 >= 256 * MG, "one reducing thread an output");
     __shared__ float part[2][MG][GF_WAVES][64][4];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, q = lane >> 4;
     const int kslice = blockIdx.y;
     static_assert(GF_WAVES * GF_KSTEPS * 32 == GF_KSPAN, "a workgroup covers GF_KSPAN of K");
-    const int k_lo = kslice * GF_KSPAN;           // this workgroup's K range starts here
-    const int k_hi = (k_lo + GF_KSPAN < K) ? k_lo + GF_KSPAN : K;
-    const int s0 = wave * GF_KSTEPS;
+    const int k_lo = kslice * kspan;              // this workgroup's K range starts here
+    const int k_hi = (k_lo + kspan < K) ? k_lo + kspan : K;
+    const int s0 = wave * ks;
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     const int k8_first = k_lo >> 3, k8_last = (k_hi >> 3) - 1;
     int k8c[GF_KSTEPS];
@@ -42,8 +45,8 @@ gemm_ksplit_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* _
 #pragma unroll
     for (int u = 0; u < GF_KSTEPS; ++u) {
         const int k8 = k8_first + (s0 + u) * 4 + q;
-        kok[u] = k8 <= k8_last;
-        k8c[u] = kok[u] ? k8 : k8_last;
+        kok[u] = u < ks && k8 <= k8_last;
+        k8c[u] = kok[u] ? k8 : (u == 0 ? k8_last : k8c[0]);
     }
     // the first W tile is on its way before anything else (after the X fragments where the activation of
     // two row groups needs the registers meanwhile)
@@ -160,6 +163,7 @@ extern "C" int ilm_gemm_ksplit(void* C, int out_dtype, int ldc, long c_part_stri
     ILM_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && lda % 8 == 0 && lda >= (act ? 2 * K : K),
                 "gemm_ksplit: X and W rows must be 16-byte aligned, X rows %d long", act ? 2 * K : K);
     const int ntiles = (N + 15) / 16;
+    const int kspan = ((K + kb - 1) / kb + 31) / 32 * 32;   // K spread evenly over the parts
     int gx = gf_num_cus() / kb;
     if (gx < 1) gx = 1;
     if (gx > ntiles) gx = ntiles;
@@ -167,7 +171,7 @@ extern "C" int ilm_gemm_ksplit(void* C, int out_dtype, int ldc, long c_part_stri
 #define KS_LAUNCH_(WV, KS, MGR, ACT, TC)                                                                       \
     gemm_ksplit_kernel<WV, KS, MGR, ACT, TC><<<grid, WV * 64, 0, stream>>>(                                    \
         (TC*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha, ntiles,      \
-        (size_t)c_part_stride)
+        (size_t)c_part_stride, kspan, (kspan / 32 + WV - 1) / WV)
 #define KS_LAUNCH(ACT, TC)                                   \
     if (M <= 16) KS_LAUNCH_(16, 8, 1, ACT, TC);              \
     else KS_LAUNCH_(8, 16, 2, ACT, TC)

@@ -31,21 +31,25 @@ gemm_qkv_rope_kernel(bf16* __restrict__ Q, const bf16* __restrict__ X, const bf1
                      const bf16* __restrict__ bias, int M, int K, int lda, int ldw, int ldq,
                      const int* __restrict__ pos, const float* __restrict__ cosT, const float* __restrict__ sinT,
                      bf16* __restrict__ kc, bf16* __restrict__ vc, const int* __restrict__ slots, int nh, int nkv,
-                     int d, int page, int n_units, int pairs_per_unit) {
+                     int d, int page, int n_units, int pairs_per_unit, int ks) {
+    // ks <= KSTEPS: k-steps a wave really takes (K spread evenly over the waves); its other slots load
+    // its first address again (a cache hit, no branch around the loads) and multiply by zeros
     static_assert(WAVES * 64 >= 256 * MG, "one reducing thread an output");
     __shared__ float part[2][MG][WAVES][64][4];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, q = lane >> 4;
-    const int s0 = wave * KSTEPS;
+    const int s0 = wave * ks;
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     const int k8_last = (K >> 3) - 1;
     const int half = d >> 1;
     uint4 xf[MG][KSTEPS];
     int k8c[KSTEPS];
+    bool kok[KSTEPS];
 #pragma unroll
     for (int u = 0; u < KSTEPS; ++u) {
         const int k8 = (s0 + u) * 4 + q;
-        k8c[u] = k8 < k8_last ? k8 : k8_last;
+        kok[u] = u < ks && k8 <= k8_last;
+        k8c[u] = kok[u] ? k8 : (u == 0 ? k8_last : k8c[0]);
     }
 #pragma unroll
     for (int g = 0; g < MG; ++g) {
@@ -54,7 +58,7 @@ gemm_qkv_rope_kernel(bf16* __restrict__ Q, const bf16* __restrict__ X, const bf1
 #pragma unroll
         for (int u = 0; u < KSTEPS; ++u) {
             const uint4 v = xp[k8c[u]];
-            xf[g][u] = ((s0 + u) * 4 + q <= k8_last && row < M) ? v : zero;   // zero fragments make the clamped W loads harmless
+            xf[g][u] = (kok[u] && row < M) ? v : zero;   // zero fragments make the clamped W loads harmless
         }
     }
     // pair p: rows hs*d + i and hs*d + i + d/2 with hs = p / (d/2), i = p % (d/2)
@@ -179,7 +183,7 @@ extern "C" int ilm_gemm_qkv_rope(void* Q, int ldq, const void* X, int lda, const
         gemm_qkv_rope_kernel<WV, KS, MGR><<<grid, WV * 64, 0, stream>>>(                                            \
             (bf16*)Q, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, K, lda, ldw, ldq, (const int*)pos, \
             (const float*)cosT, (const float*)sinT, (bf16*)kc, (bf16*)vc, (const int*)slots, nh, nkv, d, page, \
-            n_units, ppu);                                                                                     \
+            n_units, ppu, (ksteps + WV - 1) / WV);                                                             \
     }
     if (M > 16) {
         if (ksteps <= 8 * 4) QR_CASE(8, 4, 2)

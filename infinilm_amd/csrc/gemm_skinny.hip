@@ -126,20 +126,24 @@ template <int WAVES, int KSTEPS, int MG, typename TC>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_resident_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
                             const bf16* __restrict__ bias, int M, int N, int K, int lda, int ldw, int ldc,
-                            float alpha, int ntiles) {
+                            float alpha, int ntiles, int ks) {
+    // ks <= KSTEPS: k-steps a wave really takes (K spread evenly over the waves); its other slots load
+    // its first address again (a cache hit, no branch around the loads) and multiply by zeros
     static_assert(WAVES * 64 >= 256 * MG, "one reducing thread an output");
     __shared__ float part[2][MG][WAVES][64][4];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, q = lane >> 4;
-    const int s0 = wave * KSTEPS;
+    const int s0 = wave * ks;
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     const int k8_last = (K >> 3) - 1;
     uint4 xf[MG][KSTEPS];
     int k8c[KSTEPS];
+    bool kok[KSTEPS];
 #pragma unroll
     for (int u = 0; u < KSTEPS; ++u) {
         const int k8 = (s0 + u) * 4 + q;
-        k8c[u] = k8 < k8_last ? k8 : k8_last;
+        kok[u] = u < ks && k8 <= k8_last;
+        k8c[u] = kok[u] ? k8 : (u == 0 ? k8_last : k8c[0]);
     }
 #pragma unroll
     for (int g = 0; g < MG; ++g) {
@@ -149,7 +153,7 @@ gemm_skinny_resident_kernel(TC* __restrict__ C, const bf16* __restrict__ X, cons
         for (int u = 0; u < KSTEPS; ++u) {
             const uint4 v = xp[k8c[u]];
             // zero fragments beyond K or beyond M make the clamped W loads harmless
-            xf[g][u] = ((s0 + u) * 4 + q <= k8_last && row < M) ? v : zero;
+            xf[g][u] = (kok[u] && row < M) ? v : zero;
         }
     }
     uint4 a[KSTEPS];
@@ -200,28 +204,31 @@ gemm_skinny_resident_kernel(TC* __restrict__ C, const bf16* __restrict__ X, cons
 }
 
 // The fused gate/up projection of a feed-forward with the SwiGLU in its epilogue (few rows of X):
-// W holds the gate rows [0, I) and the up rows [I, 2I).  A workgroup multiplies the gate tile and
-// the up tile of the same 16 outputs one after the other; the thread that reduces output (m, n) of
-// the first also reduces (m, n) of the second and stores act[m, n] = silu(gate) * up.  The
-// intermediate [M, 2I] never goes to memory and the following projection reads plain rows.
-// Gate and up are rounded to bfloat16 before the activation, as the unfused path stores them.
+// W holds the gate rows [0, I) and the up rows [I, 2I).  A tile of 16 W rows is the gate rows and the
+// up rows of the same 8 outputs, so the thread that reduces gate (m, n) also reduces up (m, n) and
+// stores act[m, n] = silu(gate) * up.  The intermediate [M, 2I] never goes to memory and the
+// following projection reads plain rows.  Gate and up are rounded to bfloat16 before the
+// activation, as the unfused path stores them.
 template <int WAVES, int KSTEPS, int MG>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_gateup_swiglu_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
-                          const bf16* __restrict__ bias, int M, int I, int K, int lda, int ldw, int ldc, int ntiles) {
-    static_assert(WAVES * 64 >= 256 * MG, "one reducing thread an output");
+                          const bf16* __restrict__ bias, int M, int I, int K, int lda, int ldw, int ldc, int ntiles,
+                          int ks) {
+    static_assert(WAVES * 64 >= 128 * MG, "one reducing thread an output");
     __shared__ float part[2][MG][WAVES][64][4];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, q = lane >> 4;
-    const int s0 = wave * KSTEPS;
+    const int s0 = wave * ks;
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     const int k8_last = (K >> 3) - 1;
     uint4 xf[MG][KSTEPS];
     int k8c[KSTEPS];
+    bool kok[KSTEPS];
 #pragma unroll
     for (int u = 0; u < KSTEPS; ++u) {
         const int k8 = (s0 + u) * 4 + q;
-        k8c[u] = k8 < k8_last ? k8 : k8_last;
+        kok[u] = u < ks && k8 <= k8_last;
+        k8c[u] = kok[u] ? k8 : (u == 0 ? k8_last : k8c[0]);
     }
 #pragma unroll
     for (int g = 0; g < MG; ++g) {
@@ -230,7 +237,99 @@ gemm_gateup_swiglu_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, cons
 #pragma unroll
         for (int u = 0; u < KSTEPS; ++u) {
             const uint4 v = xp[k8c[u]];
-            xf[g][u] = ((s0 + u) * 4 + q <= k8_last && row < M) ? v : zero;
+            xf[g][u] = (kok[u] && row < M) ? v : zero;
+        }
+    }
+    // this lane's W row of tile t: rows 0..7 of the tile are gate rows 8 t .. 8 t + 7, rows 8..15 the up rows
+    auto w_row = [&](int t) -> const uint4* {
+        const int n = (t * 8 + (r & 7) < I) ? t * 8 + (r & 7) : I - 1;
+        return reinterpret_cast<const uint4*>(W + (size_t)(n + (r >> 3) * I) * ldw);
+    };
+    uint4 a[KSTEPS];
+    int tile = blockIdx.x;
+    if (tile < ntiles) {
+        const uint4* wp = w_row(tile);
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
+    }
+    // the reducing thread's output: row m, output j of the tile's 8
+    const int et = threadIdx.x < 128 * MG ? threadIdx.x : 0;
+    const int eg = et >> 7, m = eg * 16 + (et & 15), j = (et & 127) >> 4;
+    const int gl = (j >> 2) * 16 + (et & 15), ge = j & 3;   // lane and element of the gate sum; up: lane + 32
+    int buf = 0;
+    for (; tile < ntiles; tile += gridDim.x) {
+        f32x4 acc[MG];
+#pragma unroll
+        for (int g = 0; g < MG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u)
+#pragma unroll
+            for (int g = 0; g < MG; ++g) acc[g] = mfma16(a[u], xf[g][u], acc[g]);
+        // the next tile's rows are on their way while this one is reduced
+        const int next = tile + gridDim.x;
+        __builtin_amdgcn_sched_barrier(0);
+        if (next < ntiles) {
+            const uint4* wp = w_row(next);
+#pragma unroll
+            for (int u = 0; u < KSTEPS; ++u) a[u] = wp[k8c[u]];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 0; g < MG; ++g) *reinterpret_cast<f32x4*>(&part[buf][g][wave][lane][0]) = acc[g];
+        __syncthreads();
+        const int n = tile * 8 + j;
+        if (threadIdx.x < 128 * MG && n < I && m < M) {
+            float vg = 0.f, vu = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                vg += part[buf][eg][w][gl][ge];
+                vu += part[buf][eg][w][gl + 32][ge];
+            }
+            if (bias != nullptr) {
+                vg += to_f32(bias[n]);
+                vu += to_f32(bias[n + I]);
+            }
+            vg = to_f32(from_f32<bf16>(vg));
+            vu = to_f32(from_f32<bf16>(vu));
+            C[(size_t)m * ldc + n] = from_f32<bf16>(vg / (1.0f + expf(-vg)) * vu);
+        }
+        buf ^= 1;  // the other buffer is free: its readers passed the barrier above one tile ago
+    }
+}
+
+// The same with whole tiles: a workgroup multiplies the gate tile and the up tile of the same 16
+// outputs one after the other (16 consecutive W rows a tile: 50.5 -> 47.0 us at the 8B shape), and the
+// thread that reduces output (m, n) of the first also reduces (m, n) of the second.  For many tiles a
+// workgroup; with few, the units of two tiles leave compute units idle at the end.
+template <int WAVES, int KSTEPS, int MG>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_gateup_swiglu_pair_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
+                          const bf16* __restrict__ bias, int M, int I, int K, int lda, int ldw, int ldc, int ntiles,
+                          int ks) {
+    static_assert(WAVES * 64 >= 256 * MG, "one reducing thread an output");
+    __shared__ float part[2][MG][WAVES][64][4];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = lane & 15, q = lane >> 4;
+    const int s0 = wave * ks;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    const int k8_last = (K >> 3) - 1;
+    uint4 xf[MG][KSTEPS];
+    int k8c[KSTEPS];
+    bool kok[KSTEPS];
+#pragma unroll
+    for (int u = 0; u < KSTEPS; ++u) {
+        const int k8 = (s0 + u) * 4 + q;
+        kok[u] = u < ks && k8 <= k8_last;
+        k8c[u] = kok[u] ? k8 : (u == 0 ? k8_last : k8c[0]);
+    }
+#pragma unroll
+    for (int g = 0; g < MG; ++g) {
+        const int row = g * 16 + r;
+        const uint4* xp = reinterpret_cast<const uint4*>(X + (size_t)(row < M ? row : 0) * lda);
+#pragma unroll
+        for (int u = 0; u < KSTEPS; ++u) {
+            const uint4 v = xp[k8c[u]];
+            xf[g][u] = (kok[u] && row < M) ? v : zero;
         }
     }
     // this lane's W row of a tile's gate half (0) or up half (1)
@@ -324,7 +423,8 @@ extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void
     {                                                                                                       \
         const int grid = ntiles < num_cus() * PER_CU ? ntiles : num_cus() * PER_CU;                         \
         gemm_skinny_resident_kernel<WV, KS, MGR, TC><<<grid, WV * 64, 0, stream>>>(                         \
-            (TC*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha, ntiles); \
+            (TC*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha, ntiles, \
+            (ksteps + WV - 1) / WV);                                                                        \
     }
         // measured on MI355X at K = 4096: 8 waves of 16 k-steps (more loads in flight a wave) win where the
         // tiles are at most one a compute unit (o projection, 9.1 against 10.2 us) or many (gate/up 47.8
@@ -393,12 +493,20 @@ extern "C" int ilm_gemm_gateup_swiglu(void* C, int ldc, const void* X, int lda, 
     ILM_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_gateup_swiglu: operands must be 16-byte aligned");
     const int ksteps = (K + 31) / 32;
     ILM_REQUIRE(ksteps <= (M <= 16 ? 16 * 16 : 8 * 16), "gemm_gateup_swiglu: K=%d is beyond %d", K, M <= 16 ? 8192 : 4096);
-    const int ntiles = (I + 15) / 16;
-#define GU_CASE(WV, KS, MGR, PER_CU)                                                                        \
+    // whole tiles in pairs where every workgroup gets at least two pairs, else tiles of 8 + 8 rows
+    const bool pairs = (I + 15) / 16 >= 2 * num_cus();
+    const int ntiles = pairs ? (I + 15) / 16 : (I + 7) / 8;
+#define GU_LAUNCH(KERNEL, WV, KS, MGR, PER_CU)                                                              \
     {                                                                                                       \
         const int grid = ntiles < num_cus() * PER_CU ? ntiles : num_cus() * PER_CU;                         \
-        gemm_gateup_swiglu_kernel<WV, KS, MGR><<<grid, WV * 64, 0, stream>>>(                               \
-            (bf16*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, I, K, lda, ldw, ldc, ntiles);   \
+        KERNEL<WV, KS, MGR><<<grid, WV * 64, 0, stream>>>(                                                  \
+            (bf16*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, I, K, lda, ldw, ldc, ntiles,    \
+            (ksteps + WV - 1) / WV);                                                                        \
+    }
+#define GU_CASE(WV, KS, MGR, PER_CU)                                                       \
+    {                                                                                      \
+        if (pairs) GU_LAUNCH(gemm_gateup_swiglu_pair_kernel, WV, KS, MGR, PER_CU)          \
+        else GU_LAUNCH(gemm_gateup_swiglu_kernel, WV, KS, MGR, PER_CU)                     \
     }
     if (M > 16) {
         if (ksteps <= 8 * 4) GU_CASE(8, 4, 2, 2)
@@ -409,6 +517,7 @@ extern "C" int ilm_gemm_gateup_swiglu(void* C, int ldc, const void* X, int lda, 
     else if (ksteps <= 8 * 8) GU_CASE(8, 8, 1, 2)
     else if (ksteps <= 8 * 16) GU_CASE(8, 16, 1, 2)
     else GU_CASE(16, 16, 1, 1)
+#undef GU_LAUNCH
 #undef GU_CASE
     ILM_LAUNCH_CHECK("gemm_gateup_swiglu");
     return 0;

@@ -294,7 +294,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     # projection 22 -> 17 and 25 -> 19; up to 64 rows the library and a one-part sum are as fast)
     if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS:
         return _gemm_mid(a, w, K, False)
-    if fast and aligned and plain and allow_parts and out is None and M <= max(16, FEW_ROWS) and K > 2 * KSPLIT_SPAN and USE_KSPLIT:
+    if fast and aligned and plain and allow_parts and out is None and M <= max(16, FEW_ROWS) and K > KSPLIT_SPAN and USE_KSPLIT:
         kb = -(-K // KSPLIT_SPAN)
         parts = torch.empty((kb, M, N), dtype=F32, device=a.device)
         _run("ilm_gemm_ksplit", parts.data_ptr(), _DT[F32], N, M * N, kb, w.data_ptr(), w.stride(0), None, 1.0,
