@@ -99,7 +99,8 @@ def main(argv=None) -> int:
     llm = LLM(model_path=model_path, dtype=cfg.dtype, max_batch_size=max(c["batch_size"] for c in cases),
               num_blocks=max(need, 1), block_size=page, enable_graph=cfg.enable_graph,
               skip_load=cfg.skip_load or cfg.random_weights, max_num_batched_tokens=cfg.max_num_batched_tokens,
-              chunk_size=cfg.chunk_size, admission=cfg.admission, seed=cfg.seed)
+              chunk_size=cfg.chunk_size, admission=cfg.admission, seed=cfg.seed,
+              enable_prefix_caching=cfg.enable_prefix_caching)
     sp_kwargs = dict(temperature=cfg.temperature, top_k=cfg.top_k, top_p=cfg.top_p)
     try:
         if cfg.warmup:
@@ -107,8 +108,8 @@ def main(argv=None) -> int:
             for c in cases:   # also records the HIP graphs of each batch size
                 run_case(llm, dict(c, output_len=min(c["output_len"], 4)), cfg.seed, sp_kwargs)
             print("=================== warmup done ====================", flush=True)
-        for c in cases:
-            print(json.dumps(run_case(llm, c, cfg.seed + 1, sp_kwargs)), flush=True)
+        for i, c in enumerate(cases):   # prompts of their own for every case: no case finds another's pages
+            print(json.dumps(run_case(llm, c, cfg.seed + 1 + 1000 * (i + 1), sp_kwargs)), flush=True)
     finally:
         llm.close()
     return 0

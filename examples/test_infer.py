@@ -4,6 +4,7 @@ reference's examples/test_infer.py.
     python examples/test_infer.py --model DIR [--dtype bfloat16] [--batch-size 4]
         [--prompt "How are you" | --prompt-ids 1,5,9] [--max-new-tokens 64]
         [--top-k 1 --top-p 1.0 --temperature 1.0] [--num-blocks 512 --block-size 256]
+        [--disable-prefix-caching]
 """
 import logging
 import os
@@ -24,7 +25,8 @@ def main(argv=None) -> int:
                 num_blocks=cfg.num_blocks or None, block_size=cfg.block_size, temperature=cfg.temperature, top_k=cfg.top_k,
                 top_p=cfg.top_p, enable_graph=cfg.enable_graph, attn_backend=cfg.attn,
                 skip_load=cfg.skip_load or cfg.random_weights, max_num_batched_tokens=cfg.max_num_batched_tokens,
-                chunk_size=cfg.chunk_size, admission=cfg.admission, seed=cfg.seed)
+                chunk_size=cfg.chunk_size, admission=cfg.admission, seed=cfg.seed,
+                enable_prefix_caching=cfg.enable_prefix_caching)
     sp = SamplingParams(temperature=cfg.temperature, top_p=cfg.top_p, top_k=cfg.top_k, max_tokens=cfg.max_new_tokens,
                         ignore_eos=cfg.ignore_eos)
     t1 = time.time()

@@ -10,11 +10,21 @@ the whole prompt at admission, go straight back to the free list when a request 
 has passed them, and cache entries whose mixers keep all keys and those that keep a window form
 groups with page pools and block tables of their own.
 
+Prefix sharing (`prefix_caching=True`; the reference's python/infinilm/llm/prefix_cache.py and
+cache_manager.py:136-156, scheduler.py:158-164,503-523): a page all of whose tokens have been
+computed is published under a key chained over the tokens of the whole prefix; a request admitted
+with its tokens takes the longest run of published pages from its start (never the page of its
+last token: one token at least has to run to give logits) and begins after them.  Pages of a
+request that ends stay findable until the pool needs them.  Only where every cache entry keeps all
+keys in pages: a window's pages are given back, and a fixed-size state cannot be taken over.
+
 The control plane (this class) holds no GPU state beyond the tensors it allocates; it can be built
 with device="meta" or "cpu" and exercised without a GPU.
 """
 from __future__ import annotations
 
+import hashlib
+from array import array
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
@@ -39,6 +49,11 @@ class _Request:
     tables: List[List[int]] = field(default_factory=list)   # per group: logical page -> page id, -1 = given back
     state_slot: int = 0
     fresh: bool = True                   # no state written yet: reads start from the zero row
+    # prefix sharing: key of the last whole page, tokens since then, whole pages whose key is known;
+    # chain None = this request's tokens are unknown (committed without them): nothing is published
+    chain: Optional[bytes] = None
+    pending: List[int] = field(default_factory=list)
+    keyed_pages: int = 0
 
 
 class KVView:
@@ -60,7 +75,8 @@ class StateView:
 
 class CacheManager:
     def __init__(self, needs: Sequence, page_size: int, num_pages: int, max_requests: int,
-                 dtype: torch.dtype, device, num_pages_per_group: Optional[Dict[int, int]] = None):
+                 dtype: torch.dtype, device, num_pages_per_group: Optional[Dict[int, int]] = None,
+                 prefix_caching: bool = False):
         if page_size <= 0:
             raise CacheError(f"page size must be positive, got {page_size}")
         self.page_size = int(page_size)
@@ -103,6 +119,12 @@ class CacheManager:
         # state slots: row 0 is the permanent zero state
         self._free_slots = list(range(self.max_requests, 0, -1))
         self.requests: Dict[object, _Request] = {}
+        # prefix sharing needs one group that keeps all keys, and no state beside it
+        self.prefix_caching = bool(prefix_caching) and len(self.groups) == 1 and self.groups[0].window <= 0 \
+            and not self.state
+        self._root_key = hashlib.blake2b(b"infinilm_amd page chain 1 " + str(self.page_size).encode(), digest_size=16).digest()
+        self.prefix_hit_tokens = 0       # tokens taken over from published pages at admissions
+        self.prefix_asked_tokens = 0     # tokens of the prompts admitted with their tokens
 
     # ---- sizes ----------------------------------------------------------------------------------
     def bytes_per_token(self) -> int:
@@ -121,18 +143,65 @@ class CacheManager:
     def stats(self) -> dict:
         return {"requests": len(self.requests),
                 "groups": [{"window": g.window, "entries": len(g.entries), "pages": g.pool.num_pages,
-                            "free": g.pool.num_free, "high_water": g.pool.high_water} for g in self.groups],
-                "state_slots_free": len(self._free_slots)}
+                            "free": g.pool.num_free, "idle": g.pool.num_idle, "evictions": g.pool.evictions,
+                            "high_water": g.pool.high_water} for g in self.groups],
+                "state_slots_free": len(self._free_slots),
+                "prefix_caching": self.prefix_caching, "prefix_hit_tokens": self.prefix_hit_tokens,
+                "prefix_asked_tokens": self.prefix_asked_tokens}
+
+    # ---- keys of whole pages ----------------------------------------------------------------------
+    def _page_key(self, parent: bytes, tokens: Sequence[int]) -> bytes:
+        """Key of a whole page: a hash over the key of the page before it and its own tokens, so it
+        stands for the whole prefix."""
+        return hashlib.blake2b(parent + array("i", tokens).tobytes(), digest_size=16).digest()
+
+    def _matching_pages(self, tokens: Sequence[int]):
+        """(pages, key of the last one) of the longest published run from the start of `tokens` that
+        leaves at least the last token to be computed."""
+        pool = self.groups[0].pool
+        ps = self.page_size
+        pages, key = [], self._root_key
+        for i in range((len(tokens) - 1) // ps):
+            k = self._page_key(key, tokens[i * ps:(i + 1) * ps])
+            page = pool.lookup(k)
+            if page is None:
+                break
+            pages.append(page)
+            key = k
+        return pages, key
+
+    def peek_prefix(self, tokens: Sequence[int]):
+        """(tokens an admission with these tokens would take over from published pages, how many of those
+        pages are idle now and would leave the pages that can be given out); nothing is pinned."""
+        if not self.prefix_caching:
+            return 0, 0
+        pages = self._matching_pages(tokens)[0]
+        pool = self.groups[0].pool
+        return len(pages) * self.page_size, sum(1 for p in pages if pool.refs(p) == 0)
 
     # ---- requests -------------------------------------------------------------------------------
-    def admit(self, req_id) -> None:
+    def admit(self, req_id, tokens: Optional[Sequence[int]] = None) -> int:
+        """A new request.  With prefix sharing and the request's `tokens` (all that are known), it takes
+        over the published pages that hold its beginning; returns how many tokens they cover: the
+        request's length, from which its first step goes on."""
         if req_id in self.requests:
             raise CacheError(f"request {req_id!r} is already admitted")
         if not self._free_slots:
             raise CacheError(f"no state slot free for request {req_id!r} ({self.max_requests} requests at most)")
         r = _Request(tables=[[] for _ in self.groups], state_slot=self._free_slots.pop())
+        if self.prefix_caching and tokens is not None:
+            pages, key = self._matching_pages(tokens)
+            pool = self.groups[0].pool
+            for p in pages:
+                pool.share(p)
+            r.tables[0] = list(pages)
+            r.length = r.reserved = len(pages) * self.page_size
+            r.chain, r.keyed_pages = key, len(pages)
+            self.prefix_hit_tokens += r.length
+            self.prefix_asked_tokens += len(tokens)
         self.requests[req_id] = r
         self.version += 1
+        return r.length
 
     def has(self, req_id) -> bool:
         return req_id in self.requests
@@ -174,13 +243,20 @@ class CacheManager:
             table.extend(g.pool.take(n))
         r.reserved = max(r.reserved, r.length + n_new)
 
-    def commit(self, req_id, n_new: int) -> None:
-        """`n_new` tokens have been written; give back the pages a window has passed."""
+    def commit(self, req_id, n_new: int, tokens: Optional[Sequence[int]] = None) -> None:
+        """`n_new` tokens have been written; give back the pages a window has passed.  With prefix
+        sharing, `tokens` (the n_new token ids) let the pages they complete be published; a commit
+        without them ends the publishing for this request."""
         r = self.requests[req_id]
         if r.length + n_new > r.reserved:
             raise CacheError(f"request {req_id!r}: commit of {n_new} tokens beyond what was reserved")
         r.length += n_new
         r.fresh = False
+        if self.prefix_caching and r.chain is not None:
+            if tokens is None or len(tokens) != n_new:
+                r.chain, r.pending = None, []
+            else:
+                self._publish(r, tokens)
         for g, table in zip(self.groups, r.tables):
             first = self._first_needed_page(g, r.length)  # the next query sits at position `length`
             for i in range(min(first, len(table))):
@@ -204,13 +280,27 @@ class CacheManager:
         r = self.requests[req_id]
         return (0 if r.fresh else r.state_slot), r.state_slot
 
+    def _publish(self, r: _Request, tokens: Sequence[int]) -> None:
+        ps = self.page_size
+        pool = self.groups[0].pool
+        r.pending.extend(tokens)
+        while len(r.pending) >= ps:
+            key = self._page_key(r.chain, r.pending[:ps])
+            pool.publish(r.tables[0][r.keyed_pages], key)   # False: the same content is already there; ours stays private
+            r.chain = key
+            r.keyed_pages += 1
+            del r.pending[:ps]
+
     def release(self, req_id) -> None:
-        """The request is over (or preempted): all its pages and its slot go back."""
+        """The request is over (or preempted): all its pages and its slot go back.  Published pages go
+        last page first, so that of a run the end loses its content before the beginning."""
         r = self.requests.pop(req_id, None)
         if r is None:
             raise CacheError(f"request {req_id!r} is not admitted (released twice?)")
         for g, table in zip(self.groups, r.tables):
-            g.pool.give_back([p for p in table if p >= 0])
+            pages = [p for p in table if p >= 0]
+            g.pool.give_back([p for p in pages if not g.pool.is_published(p)])
+            g.pool.give_back([p for p in reversed(pages) if g.pool.is_published(p)])
         self._free_slots.append(r.state_slot)
         self.version += 1
 
@@ -218,9 +308,18 @@ class CacheManager:
         """No page lost, none held twice: the pages in the block tables are exactly the held ones."""
         for gi, g in enumerate(self.groups):
             g.pool.check()
-            held = [p for r in self.requests.values() for p in r.tables[gi] if p >= 0]
-            if len(held) != len(set(held)):
-                raise CacheError(f"group {gi}: a page is in two block tables")
+            held: Dict[int, int] = {}
+            for r in self.requests.values():
+                pages = [p for p in r.tables[gi] if p >= 0]
+                if len(pages) != len(set(pages)):
+                    raise CacheError(f"group {gi}: a page is twice in one block table")
+                for p in pages:
+                    held[p] = held.get(p, 0) + 1
+            for p, n in held.items():
+                if g.pool.refs(p) != n:
+                    raise CacheError(f"group {gi}: page {p} is in {n} block tables and has {g.pool.refs(p)} owners")
+                if n > 1 and not self.prefix_caching:
+                    raise CacheError(f"group {gi}: page {p} is in two block tables")
             if len(held) != g.pool.num_held:
                 raise CacheError(f"group {gi}: {g.pool.num_held} pages held, {len(held)} in block tables")
         slots = [r.state_slot for r in self.requests.values()]

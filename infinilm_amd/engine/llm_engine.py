@@ -77,7 +77,7 @@ class LLMEngine:
         done = self.scheduler.update(out, sampled)
         c = self.counters
         c["steps"] += 1
-        if len(tokens) != len(out.entries) or out.entries[0].num_tokens != 1:   # not a step of decoded tokens alone
+        if not out.decode_only:
             c["prompt_tokens"] += sum(e.num_tokens for e in out.entries if e.start < e.request.get_prompt_length())
         c["generated_tokens"] += len(tokens)
         c["step_s"] += t2 - t1

@@ -73,10 +73,12 @@ def pages_that_fit(model: CausalLM, page_size: int, memory_fraction: float = 0.9
 
 
 def make_runner(model: CausalLM, num_pages: Optional[int], page_size: int, max_requests: int,
-                enable_graph: bool = False) -> StepRunner:
-    """`num_pages=None`: as many pages as fit into the free device memory (see `pages_that_fit`)."""
+                enable_graph: bool = False, prefix_caching: bool = False) -> StepRunner:
+    """`num_pages=None`: as many pages as fit into the free device memory (see `pages_that_fit`).
+    `prefix_caching`: whole pages of computed tokens are published for later requests with the same
+    beginning (where the model's cache entries allow it: `runner.cache.prefix_caching` tells)."""
     if num_pages is None:
         num_pages = pages_that_fit(model, page_size)
     cache = CacheManager(model.cache_needs, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
-                         dtype=model.dtype, device=model.device)
+                         dtype=model.dtype, device=model.device, prefix_caching=prefix_caching)
     return StepRunner(model, cache, enable_graph=enable_graph)

@@ -57,6 +57,7 @@ class InferenceRequest:
         self.output_token_ids: List[int] = []
         self.generated_text = ""
         self.num_computed_tokens = 0        # tokens whose keys are in the cache
+        self.num_cached_tokens = 0          # of these, taken over from published pages at the last admission
         self.status = RequestStatus.WAITING
         self.finish_reason: Optional[FinishReason] = None
         self.error: Optional[str] = None

@@ -42,6 +42,7 @@ class ScheduledEntry:
 class SchedulerOutput:
     entries: List[ScheduledEntry] = field(default_factory=list)
     preempted: List[InferenceRequest] = field(default_factory=list)
+    decode_only: bool = False    # known to hold nothing but decoded tokens (no token of a prompt)
 
     @property
     def num_tokens(self) -> int:
@@ -116,12 +117,16 @@ class Scheduler:
         held = len(self.cache.table(req.request_id, 0)) if self.cache.has(req.request_id) and self.cache.groups else 0
         return max(0, self._pages_for(total) - held)
 
-    def _can_admit(self, req: InferenceRequest, first_portion: int, promised: List[int]) -> bool:
+    def _can_admit(self, req: InferenceRequest, first_portion_end: int, promised: List[int],
+                   shared_pages: int = 0, shared_idle: int = 0) -> bool:
+        """`first_portion_end`: tokens cached after the request's first step.  `shared_pages` of them it
+        takes over from published pages; `shared_idle` of those are idle now, so taking them over
+        leaves that many fewer pages to give out."""
         if self.policy == "reserve_full":
             need = self._pages_for(min(req.get_prompt_length() + req.sampling_params.max_tokens, self.max_positions))
-            need += sum(self._worst_case_pages(r) for r in self.running)
+            need += sum(self._worst_case_pages(r) for r in self.running) - shared_pages + shared_idle
             return all(need <= g.pool.num_free for g in self.cache.groups)
-        need = self._pages_for(first_portion)
+        need = self._pages_for(first_portion_end) - shared_pages + shared_idle
         return all(p + need <= g.pool.num_free for p, g in zip(promised, self.cache.groups))
 
     def _preempt(self, victim: InferenceRequest, out: SchedulerOutput) -> None:
@@ -145,7 +150,7 @@ class Scheduler:
         for g in self.cache.groups:
             if g.pool.num_free < R:
                 return None
-        out = SchedulerOutput()
+        out = SchedulerOutput(decode_only=True)
         entries = out.entries
         for req in running:            # `running` is in order of admission
             start = req.num_computed_tokens
@@ -221,11 +226,14 @@ class Scheduler:
             req = self.waiting[0]
             if req in out.preempted:          # just made room for an older request: wait a step
                 break
-            n = min(req.num_known_tokens(), self.chunk_size, budget)
-            if not self._can_admit(req, n, promised):
+            # with prefix sharing the request begins after the published pages that hold its beginning
+            tokens = req.all_token_ids() if self.cache.prefix_caching else None
+            hit, idle = self.cache.peek_prefix(tokens) if tokens is not None else (0, 0)
+            n = min(req.num_known_tokens() - hit, self.chunk_size, budget)
+            if not self._can_admit(req, hit + n, promised, hit // self.cache.page_size, idle):
                 break
             self.waiting.popleft()
-            self.cache.admit(req.request_id)
+            req.num_computed_tokens = req.num_cached_tokens = self.cache.admit(req.request_id, tokens)
             req.status = RequestStatus.RUNNING
             req.admission_index = self._admissions
             self._admissions += 1

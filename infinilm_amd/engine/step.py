@@ -288,7 +288,7 @@ class StepRunner:
         batch.taps = taps
         logits = self.model.forward(batch, self.cache)
         for e in entries:
-            self.cache.commit(e.req_id, len(e.tokens))
+            self.cache.commit(e.req_id, len(e.tokens), e.tokens)
         self.steps += 1
         self.tokens += batch.T
         return logits
@@ -346,7 +346,7 @@ class StepRunner:
                     raise RuntimeError("a decode step does not fit the graph captured for its size")
         graph.replay()
         for e in entries:
-            cache.commit(e.req_id, 1)
+            cache.commit(e.req_id, 1, e.tokens)
         self.steps += 1
         self.tokens += R
         self._prepare_next_decode(entries)

@@ -39,19 +39,20 @@ class LLM:
     temperature / top_p / top_k   defaults of requests that bring no SamplingParams
     max_num_batched_tokens / chunk_size   token budget of a step / longest portion of a prompt
     admission       "optimistic" (preempt when pages run out) | "reserve_full" (the reference's check)
+    enable_prefix_caching   whole pages of computed tokens stay findable for later requests that begin
+                    with the same tokens (the reference's default; off where a model's cache entries
+                    keep a window or a state of their own)
     """
 
     def __init__(self, model_path, device: str = "cuda", dtype: Optional[str] = None, cache_type: str = "paged",
                  max_batch_size: int = 16, max_tokens: int = 4096, num_blocks: Optional[int] = 512, block_size: int = 256,
                  max_cache_len: Optional[int] = None, temperature: float = 1.0, top_p: float = 0.8, top_k: int = 1,
                  enable_graph: bool = False, attn_backend: str = "default", skip_load: bool = False,
-                 enable_prefix_caching: bool = False, max_num_batched_tokens: Optional[int] = None,
+                 enable_prefix_caching: bool = True, max_num_batched_tokens: Optional[int] = None,
                  chunk_size: Optional[int] = None, admission: str = "optimistic", seed: int = 0,
                  random_weights: bool = False, random_std: float = 0.02, tokenizer=None):
         if cache_type != "paged":
             raise ValueError("only the paged cache exists here (cache_type='paged')")
-        if enable_prefix_caching:
-            raise NotImplementedError("prefix caching is not built; pass enable_prefix_caching=False")
         if attn_backend not in ("default", "paged-attn"):
             raise ValueError("one attention backend exists here: 'default' (= 'paged-attn')")
         dev = "cuda:0" if device in ("cuda", "auto", "hip") else device
@@ -68,7 +69,7 @@ class LLM:
         self.model = model
         self.default_sampling = SamplingParams(temperature=temperature, top_p=top_p, top_k=top_k, max_tokens=max_tokens)
         runner = make_runner(model, num_pages=num_blocks, page_size=block_size, max_requests=max_batch_size,
-                             enable_graph=enable_graph)
+                             enable_graph=enable_graph, prefix_caching=enable_prefix_caching)
         if max_num_batched_tokens is None:
             env = os.environ.get("INFINILM_MAX_NUM_BATCHED_TOKENS")  # python/infinilm/llm/llm.py:99-102
             max_num_batched_tokens = int(env) if env else model.spec.max_positions

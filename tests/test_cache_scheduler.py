@@ -145,6 +145,167 @@ def test_no_page_lost_held_twice_or_freed_twice_under_random_orders(seed):
     assert all(g.pool.num_free == 24 for g in c.groups)
 
 
+def test_published_pages_are_shared_idle_and_taken_last():
+    pool = PagePool(4)
+    a, b = pool.take(2)
+    assert pool.publish(a, b"k1") and pool.publish(b, b"k2") and pool.lookup(b"k1") == a
+    with pytest.raises(CacheError, match="published twice"):
+        pool.publish(a, b"k3")
+    c = pool.take(1)[0]
+    assert not pool.publish(c, b"k1") and not pool.is_published(c)     # the same content is there already
+    pool.share(a)
+    assert pool.refs(a) == 2
+    with pytest.raises(CacheError, match="not published"):
+        pool.share(c)
+    pool.give_back([b, a])                 # b idle, a still held once
+    assert pool.num_idle == 1 and pool.num_free == 2 and pool.lookup(b"k2") == b
+    pool.give_back([a])
+    assert pool.num_idle == 2 and pool.num_held == 1
+    pool.check()
+    pool.share(b)                          # an idle page found again is held again
+    assert pool.num_idle == 1 and pool.refs(b) == 1
+    got = pool.take(2)                     # the free page first, then the idle one, which loses its content
+    assert got == [3, a] and pool.lookup(b"k1") is None and pool.evictions == 1 and not pool.is_published(a)
+    with pytest.raises(OutOfPages):
+        pool.take(1)
+    pool.give_back([got[0]])
+    with pytest.raises(CacheError, match="nobody holds"):
+        pool.publish(got[0], b"x")
+    pool.check()
+
+
+def _shared_cache(num_pages=10, page_size=4, **kw):
+    return CacheManager([PagedKV(1, 4), PagedKV(2, 8)], page_size=page_size, num_pages=num_pages, max_requests=6,
+                        dtype=torch.float32, device="cpu", prefix_caching=True, **kw)
+
+
+def test_a_request_takes_over_the_published_pages_of_its_beginning():
+    c = _shared_cache()
+    assert c.prefix_caching
+    toks = list(range(100, 111))            # 11 tokens: two whole pages and three
+    assert c.admit("a", toks) == 0 and c.peek_prefix(toks) == (0, 0)
+    c.reserve("a", 11)
+    c.commit("a", 6, toks[:6])              # one whole page computed
+    assert c.peek_prefix(toks) == (4, 0)
+    c.commit("a", 5, toks[6:])
+    assert c.peek_prefix(toks) == (8, 0) and c.table("a", 0) == [0, 1, 2]
+    # the same beginning: the whole pages are shared, the rest is the request's own
+    assert c.admit("b", toks[:8] + [7, 7, 7]) == 8
+    assert c.table("b", 0) == [0, 1] and c.length("b") == 8 and c.pages_needed("b", 3) == [1]
+    c.reserve("b", 3)
+    assert c.table("b", 0) == [0, 1, 3]
+    c.check()
+    # never the page of the last token: a prompt of exactly two pages takes one over
+    assert c.peek_prefix(toks[:8]) == (4, 0) and c.peek_prefix(toks[:9]) == (8, 0) and c.peek_prefix(toks[:4]) == (0, 0)
+    # another beginning finds nothing, and a page is only found behind the pages before it
+    assert c.peek_prefix([1] + toks[1:]) == (0, 0) and c.peek_prefix([9, 9, 9, 9] + toks[4:]) == (0, 0)
+    c.release("a")                          # its shared pages stay held by b, its own last page is free again
+    assert c.free_pages() == 10 - 3 and c.groups[0].pool.num_idle == 0
+    c.release("b")
+    assert c.free_pages() == 10 and c.groups[0].pool.num_idle == 2
+    assert c.peek_prefix(toks) == (8, 2)    # still findable, and idle
+    assert c.admit("c", toks) == 8 and c.groups[0].pool.num_idle == 0
+    st = c.stats()
+    assert st["prefix_hit_tokens"] == 16 and st["prefix_asked_tokens"] == 33
+    c.release("c")
+    c.check()
+
+
+def test_idle_pages_give_way_from_the_end_of_a_run():
+    c = _shared_cache(num_pages=4)
+    toks = list(range(13))
+    c.admit("a", toks)
+    c.reserve("a", 13)
+    c.commit("a", 13, toks)
+    c.release("a")                          # three published pages idle, one free
+    assert c.groups[0].pool.num_idle == 3 and c.free_pages() == 4
+    c.admit("x")
+    c.reserve("x", 8)                       # the free page, then the end of a's run
+    assert c.peek_prefix(toks) == (8, 2)
+    c.commit("x", 8)                        # committed without tokens: nothing of x is ever published
+    c.reserve("x", 4)
+    assert c.peek_prefix(toks) == (4, 1)
+    c.check()
+    c.commit("x", 4)
+    c.release("x")
+    assert c.groups[0].pool.num_idle == 1 and c.free_pages() == 4
+    # a request whose tokens stop being told stops publishing, and says so by never being found
+    c.admit("y", [5] * 9)
+    c.reserve("y", 9)
+    c.commit("y", 4, [5] * 4)
+    c.commit("y", 5)
+    assert c.peek_prefix([5] * 9) == (4, 0)
+    c.release("y")
+    c.check()
+
+
+def test_prefix_sharing_is_off_where_a_window_or_a_state_is_kept():
+    w = CacheManager([PagedKV(1, 4), PagedKV(1, 4, window=8)], page_size=4, num_pages=8, max_requests=2,
+                     dtype=torch.float32, device="cpu", prefix_caching=True)
+    s = CacheManager([PagedKV(1, 4), FixedState((3,))], page_size=4, num_pages=8, max_requests=2,
+                     dtype=torch.float32, device="cpu", prefix_caching=True)
+    for c in (w, s):
+        assert not c.prefix_caching
+        assert c.admit("a", list(range(9))) == 0
+        c.reserve("a", 9)
+        c.commit("a", 9, list(range(9)))
+        assert c.peek_prefix(list(range(9))) == (0, 0)
+        c.release("a")
+        assert c.groups[0].pool.num_idle == 0
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_shared_pages_under_random_orders(seed):
+    """Requests drawn from a few prompts that share beginnings, admitted, advanced and released in
+    random order with few pages: owners and block tables agree at every moment, what is found under
+    a request's tokens are its own published pages, nothing is lost at the end."""
+    rng = random.Random(100 + seed)
+    c = _shared_cache(num_pages=14, page_size=4)
+    stems = [[rng.randrange(50) for _ in range(20)] for _ in range(2)]
+    live = {}
+    n_id = 0
+    for _ in range(700):
+        op = rng.random()
+        if op < 0.25 and len(live) < 5:
+            stem = rng.choice(stems)
+            toks = stem[:rng.randrange(1, 21)] + [rng.randrange(50) for _ in range(rng.randrange(0, 8))]
+            rid = f"r{n_id}"
+            n_id += 1
+            want, idle = c.peek_prefix(toks)
+            free_before = c.free_pages()
+            got = c.admit(rid, toks)
+            assert got == want and got <= len(toks) - 1 and got % 4 == 0 and c.free_pages() == free_before - idle
+            live[rid] = (toks, got)
+        elif op < 0.85 and live:
+            rid = rng.choice(list(live))
+            toks, done = live[rid]
+            n = min(rng.choice([1, 1, 2, 5, 11]), len(toks) - done)
+            if n == 0:                      # the prompt is through: a generated token
+                toks.append(rng.randrange(50))
+                n = 1
+            if c.can_reserve(rid, n):
+                c.reserve(rid, n)
+                c.commit(rid, n, toks[done:done + n])
+                live[rid] = (toks, done + n)
+                assert c.length(rid) == done + n
+        elif live:
+            rid = rng.choice(list(live))
+            c.release(rid)
+            del live[rid]
+        c.check()
+        for rid, (toks, done) in live.items():
+            # what is findable under a live request's tokens never exceeds its whole pages, and where its
+            # own pages are the published ones they are what is found
+            pages, _ = c._matching_pages(toks[:done] + [0])
+            assert len(pages) <= done // 4
+            own = c.table(rid, 0)
+            assert all(p == own[i] for i, p in enumerate(pages) if c.groups[0].pool.is_published(own[i]))
+    for rid in list(live):
+        c.release(rid)
+    c.check()
+    assert c.free_pages() == 14 and not c.requests
+
+
 # ------------------------------------------------------------------------------------------------
 # scheduler
 # ------------------------------------------------------------------------------------------------
@@ -163,8 +324,9 @@ def _run(sched, token_of=lambda req: 7, max_steps=500):
         out = sched.schedule()
         assert out.entries, "the scheduler made no progress"
         for e in out.entries:
+            assert e.start == sched.cache.length(e.request.request_id)
             sched.cache.reserve(e.request.request_id, e.num_tokens)
-            sched.cache.commit(e.request.request_id, e.num_tokens)
+            sched.cache.commit(e.request.request_id, e.num_tokens, e.request.token_slice(e.start, e.num_tokens))
         sched.update(out, {e.request.request_id: token_of(e.request) for e in out.entries if e.samples})
         sched.cache.check()
         steps.append(out)
@@ -278,10 +440,11 @@ def test_optimistic_admission_preempts_the_newest_when_pages_run_out():
     assert r.status == RequestStatus.FAILED and "no_capacity" in r.error and c2.free_pages() == 2
 
 
+@pytest.mark.parametrize("sharing", [False, True])
 @pytest.mark.parametrize("seed", range(4))
-def test_every_admitted_request_finishes_under_random_load(seed):
+def test_every_admitted_request_finishes_under_random_load(seed, sharing):
     rng = random.Random(seed)
-    c = _cache(num_pages=14, page_size=4)
+    c = _shared_cache(num_pages=14, page_size=4) if sharing else _cache(num_pages=14, page_size=4)
     s = Scheduler(c, max_num_seqs=3, max_num_batched_tokens=rng.choice([5, 9, 32]), chunk_size=rng.choice([3, 8, 64]),
                   policy=rng.choice(["optimistic", "reserve_full"]), max_positions=1000)
     reqs = [_req(f"r{i}", rng.randint(1, 25), max_tokens=rng.randint(1, 12)) for i in range(12)]
@@ -304,7 +467,9 @@ def test_every_admitted_request_finishes_under_random_load(seed):
         assert len({e.request.request_id for e in out.entries}) == len(out.entries) <= 3
         assert out.num_tokens <= s.max_num_batched_tokens
         for e in out.entries:
-            c.reserve(e.request.request_id, e.num_tokens); c.commit(e.request.request_id, e.num_tokens)
+            assert e.start == c.length(e.request.request_id)
+            c.reserve(e.request.request_id, e.num_tokens)
+            c.commit(e.request.request_id, e.num_tokens, e.request.token_slice(e.start, e.num_tokens))
         s.update(out, {e.request.request_id: 7 for e in out.entries if e.samples})
         c.check()
     assert short_plans > 0
@@ -313,6 +478,45 @@ def test_every_admitted_request_finishes_under_random_load(seed):
     assert all(r.get_num_generated_tokens() == r.sampling_params.max_tokens for r in ok)
     assert all("no_capacity" in r.error for r in reqs if r.status == RequestStatus.FAILED)
     assert c.free_pages() == 14 and not c.requests
+
+
+def test_a_later_request_begins_after_the_pages_it_shares():
+    c = _shared_cache(num_pages=8, page_size=4)
+    s = Scheduler(c, max_num_seqs=4, max_num_batched_tokens=64, max_positions=1000)
+    a = _req("a", 14, max_tokens=3)
+    s.add_request(a)
+    _run(s)
+    assert a.num_cached_tokens == 0 and c.groups[0].pool.num_idle == 4      # 14 + 3 - 1 computed tokens: 4 whole pages
+    b, d = _req("b", 14, max_tokens=2), _req("d", 9, max_tokens=2)        # the same beginnings (1, 2, 3, ...)
+    s.add_request(b)
+    s.add_request(d)
+    out = s.schedule()
+    shape = [(e.request.request_id, e.start, e.num_tokens, e.samples) for e in out.entries]
+    assert shape == [("b", 12, 2, True), ("d", 8, 1, True)]                  # never the page of the last token
+    assert b.num_cached_tokens == 12 and d.num_cached_tokens == 8
+    assert c.table("b", 0)[:2] == c.table("d", 0)[:2] and c.groups[0].pool.refs(c.table("b", 0)[0]) == 2
+    for e in out.entries:
+        c.reserve(e.request.request_id, e.num_tokens)
+        c.commit(e.request.request_id, e.num_tokens, e.request.token_slice(e.start, e.num_tokens))
+    s.update(out, {"b": 7, "d": 7})
+    _run(s)
+    c.check()
+    assert c.free_pages() == 8 and c.stats()["prefix_hit_tokens"] == 20
+    # shared pages are not counted twice: with 8 pages, two requests of 7 pages' length run together
+    # when six of the pages are the same
+    c2 = _shared_cache(num_pages=8, page_size=4)
+    s2 = Scheduler(c2, max_num_seqs=4, max_num_batched_tokens=64, max_positions=1000)
+    first = _req("p", 25, max_tokens=20)
+    s2.add_request(first)
+    out = s2.schedule()
+    c2.reserve("p", 25)
+    c2.commit("p", 25, first.token_slice(0, 25))
+    s2.update(out, {"p": 7})
+    second = _req("q", 25, max_tokens=2)
+    s2.add_request(second)
+    out = s2.schedule()
+    assert [(e.request.request_id, e.start, e.num_tokens) for e in out.entries] == [("p", 25, 1), ("q", 24, 1)]
+    assert c2.free_pages() == 1 and not out.preempted
 
 
 def test_token_slice_equals_a_slice_of_all_tokens():

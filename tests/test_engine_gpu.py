@@ -46,6 +46,42 @@ def test_greedy_generation_through_the_entry_point(models, name):
     llm.close()
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_requests_that_share_a_beginning_share_its_pages(models, name):
+    """One prompt, then the same prompt with other endings, the prompt again, and a request that is
+    preempted and finds its own pages: with the published pages taken over, the tokens are the
+    plain implementation's (float32: the shared keys are bit for bit what the request would have
+    computed), and fewer tokens run."""
+    from infinilm_amd import LLM, SamplingParams
+
+    cfg, d, W = models[(name, "float32")]
+    stem = random_tokens(cfg, 37, 900)
+    prompts = [stem, stem + random_tokens(cfg, 6, 901), stem[:30] + random_tokens(cfg, 9, 902), stem, stem[:8]]
+    sp = SamplingParams(top_k=1, max_tokens=10)
+    ran = {}
+    for sharing in (True, False):
+        llm = LLM(d, dtype="float32", num_blocks=40, block_size=8, max_batch_size=2, chunk_size=16,
+                  enable_prefix_caching=sharing)
+        assert llm.engine.runner.cache.prefix_caching == sharing
+        first = llm.generate(prompt_token_ids=[prompts[0]], sampling_params=sp)
+        rest = llm.generate(prompt_token_ids=prompts[1:], sampling_params=sp)
+        for p, o in zip(prompts, first + rest):
+            assert o.outputs[0].token_ids == P.plain_greedy(cfg, W, p, 10), f"sharing {sharing}, prompt of {len(p)}"
+        st = llm.engine.stats()
+        ran[sharing] = st["prompt_tokens"]
+        if sharing:
+            # whole pages of 8 below the last token: 32 of 37+6, 24 of 30+9, 32 of 37 and 0 of 8
+            assert st["cache"]["prefix_hit_tokens"] == 32 + 24 + 32
+            reqs = list(llm.engine.requests.values())
+            assert [r.num_cached_tokens for r in reqs] == [0, 32, 24, 32, 0]
+        else:
+            assert st["cache"]["prefix_hit_tokens"] == 0
+        assert llm.engine.runner.cache.free_pages() == 40
+        llm.engine.runner.cache.check()
+        llm.close()
+    assert ran[False] - ran[True] == 32 + 24 + 32
+
+
 def test_greedy_generation_bfloat16_with_graphs(models):
     """bfloat16 with decode steps replayed from captured graphs gives the same tokens as eager
     bfloat16 steps, and the plain implementation's up to near ties."""
