@@ -375,13 +375,18 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     // PAGE64: the page size is a multiple of the tile's 64 keys, so a tile lies on one page: one page
     // lookup a tile (the same for every thread) and no clamping - keys of the page beyond the tokens'
     // reach are masked later.  Otherwise every piece finds its own page.
+    // V row of piece pc: of 16 consecutive pieces the first 8 are one row and the next 8 the row 8
+    // further on (not the next one): with rows 36 banks apart the two halves of a 16-lane store then
+    // fall on different halves of the banks
+    static_assert(ATT_TK == 64, "v_row places 8 pieces a row");
+    auto v_row = [](int pc) -> int { return (pc >> 7) * 16 + ((pc & 127) >> 4) + 8 * ((pc >> 3) & 1); };
     int koff[4], voff[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int pk = tid + i * 256 < KPIECES ? tid + i * 256 : 0;
         const int pv = tid + i * 256 < VPIECES ? tid + i * 256 : 0;
         koff[i] = (pk / (D / 8)) * D + (pk % (D / 8)) * 8;
-        voff[i] = (pv / (ATT_TK / 8)) * page + (pv % (ATT_TK / 8)) * 8;
+        voff[i] = v_row(pv) * page + (pv % (ATT_TK / 8)) * 8;
     }
     const bf16* ktile = kc;
     const bf16* vtile = vc;
@@ -397,7 +402,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     auto fetch_v = [&](int kb, int i) -> uint4 {
         if (PAGE64) return *reinterpret_cast<const uint4*>(vtile + voff[i]);
         const int pc = tid + i * 256;
-        const int drow = (pc < VPIECES ? pc : 0) / (ATT_TK / 8), kgrp = (pc < VPIECES ? pc : 0) % (ATT_TK / 8);
+        const int drow = v_row(pc < VPIECES ? pc : 0), kgrp = (pc < VPIECES ? pc : 0) % (ATT_TK / 8);
         int key0 = kb + kgrp * 8;
         if (key0 > p_last || key0 + 8 <= lo_first) key0 = lo_first & ~7;   // masked later; any valid group
         const int pg = page_of(key0);
@@ -414,7 +419,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     };
     auto stash_v = [&](int i, uint4 v) {
         const int pc = tid + i * 256;
-        if (pc < VPIECES) *reinterpret_cast<uint4*>(&Vs[pc / (ATT_TK / 8)][(pc % (ATT_TK / 8)) * 8]) = v;
+        if (pc < VPIECES) *reinterpret_cast<uint4*>(&Vs[v_row(pc)][(pc % (ATT_TK / 8)) * 8]) = v;
     };
     uint4 k0 = zero4, k1 = zero4, k2 = zero4, k3 = zero4, v0 = zero4, v1 = zero4, v2 = zero4, v3 = zero4;
 #define ATT_FETCH(kb_)                          \
