@@ -301,10 +301,18 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
                  int max_blocks, int q_stride, int out_stride, float scale_log2e, int window, int pair_base) {
     constexpr int D = D16 * 16;
     constexpr int KS = (D + 31) / 32;
-    constexpr int KROW = D + 8;         // padded rows: conflict-free 16-byte reads of 16 rows
-    constexpr int VROW = ATT_TK + 8;
-    __shared__ __attribute__((aligned(16))) bf16 Ks[ATT_TK][KROW];
-    __shared__ __attribute__((aligned(16))) bf16 Vs[D][VROW];
+    // K rows [key][d] and V rows [d][key] in LDS, read in 16-byte pieces by 16 rows x 4 lane groups.
+    // Head size 128: rows unpadded and the pieces of a row exchanged by an exclusive-or with the row's
+    // number (K: piece ^ (row & 15); V, two rows a 256-byte line: piece ^ ((row >> 1) & 7)), so the 16
+    // rows one matrix operand reads fall on 16 different 16-byte bank groups whichever lanes the
+    // hardware serves together.  Other head sizes: rows padded by 16 bytes.
+    constexpr bool SWZ = D == 128;
+    constexpr int KROW = SWZ ? D : D + 8;
+    constexpr int VROW = SWZ ? ATT_TK : ATT_TK + 8;
+    __shared__ __attribute__((aligned(16))) bf16 Ks[ATT_TK * KROW];
+    __shared__ __attribute__((aligned(16))) bf16 Vs[D * VROW];
+    auto k_at = [](int row, int piece) -> int { return row * KROW + (SWZ ? (piece ^ (row & 15)) : piece) * 8; };
+    auto v_at = [](int row, int piece) -> int { return row * VROW + (SWZ ? (piece ^ ((row >> 1) & 7)) : piece) * 8; };
     __shared__ int bt_s[ATT_BT_LDS];
     // Items (tile, head group) in descending order of length: the longest tiles (latest positions)
     // are dispatched first.  When the whole launch is resident at once (at most two workgroups a
@@ -379,7 +387,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     // further on (not the next one): with rows 36 banks apart the two halves of a 16-lane store then
     // fall on different halves of the banks
     static_assert(ATT_TK == 64, "v_row places 8 pieces a row");
-    auto v_row = [](int pc) -> int { return (pc >> 7) * 16 + ((pc & 127) >> 4) + 8 * ((pc >> 3) & 1); };
+    auto v_row = [](int pc) -> int { return SWZ ? pc >> 3 : (pc >> 7) * 16 + ((pc & 127) >> 4) + 8 * ((pc >> 3) & 1); };
     int koff[4], voff[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -415,11 +423,11 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
         // consecutive rows, which the row padding spreads over all banks.
         const int kk = pc / (D / 8);
         const int prow = (kk & 32) | ((kk & 4) << 2) | ((kk & 24) >> 1) | (kk & 3);
-        if (pc < KPIECES) *reinterpret_cast<uint4*>(&Ks[prow][(pc % (D / 8)) * 8]) = v;
+        if (pc < KPIECES) *reinterpret_cast<uint4*>(&Ks[k_at(prow, pc % (D / 8))]) = v;
     };
     auto stash_v = [&](int i, uint4 v) {
         const int pc = tid + i * 256;
-        if (pc < VPIECES) *reinterpret_cast<uint4*>(&Vs[v_row(pc)][(pc % (ATT_TK / 8)) * 8]) = v;
+        if (pc < VPIECES) *reinterpret_cast<uint4*>(&Vs[v_at(v_row(pc), pc % (ATT_TK / 8))]) = v;
     };
     uint4 k0 = zero4, k1 = zero4, k2 = zero4, k3 = zero4, v0 = zero4, v1 = zero4, v2 = zero4, v3 = zero4;
 #define ATT_FETCH(kb_)                          \
@@ -465,7 +473,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
 #pragma unroll
         for (int tau = 0; tau < 2; ++tau)
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) kf0[tau][ks] = *reinterpret_cast<const uint4*>(&Ks[tau * 16 + r][ks * 32 + qg * 8]);
+            for (int ks = 0; ks < KS; ++ks) kf0[tau][ks] = *reinterpret_cast<const uint4*>(&Ks[k_at(tau * 16 + r, ks * 4 + qg)]);
 #pragma unroll
         for (int tau = 0; tau < 2; ++tau)
 #pragma unroll
@@ -483,7 +491,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
 #pragma unroll
         for (int tau = 0; tau < 2; ++tau)
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) kf1[tau][ks] = *reinterpret_cast<const uint4*>(&Ks[32 + tau * 16 + r][ks * 32 + qg * 8]);
+            for (int ks = 0; ks < KS; ++ks) kf1[tau][ks] = *reinterpret_cast<const uint4*>(&Ks[k_at(32 + tau * 16 + r, ks * 4 + qg)]);
         // the reference point of the exponent follows the maximum lazily (see below); rare
 #define ATT_FOLLOW(S_, PRE_)                                                                               \
         {                                                                                                  \
@@ -552,7 +560,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
         ATT_FOLLOW(s1, {
             _Pragma("unroll") for (int j = 0; j < ATT_NT; ++j) lacc[j] = mfma16(ones4, pf0[j], lacc[j]);
             _Pragma("unroll") for (int db = 0; db < D16; ++db) {
-                const uint4 v = *reinterpret_cast<const uint4*>(&Vs[db * 16 + r][qg * 8]);
+                const uint4 v = *reinterpret_cast<const uint4*>(&Vs[v_at(db * 16 + r, qg)]);
                 _Pragma("unroll") for (int j = 0; j < ATT_NT; ++j) acc[j][db] = mfma16(v, pf0[j], acc[j][db]);
             }
             _Pragma("unroll") for (int j = 0; j < ATT_NT; ++j) pf0[j] = zero4;
@@ -560,7 +568,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
         constexpr int DH = (D16 + 1) / 2;   // value fragments in two halves: fewer registers live
         uint4 vf[DH];
 #pragma unroll
-        for (int db = 0; db < DH; ++db) vf[db] = *reinterpret_cast<const uint4*>(&Vs[db * 16 + r][qg * 8]);
+        for (int db = 0; db < DH; ++db) vf[db] = *reinterpret_cast<const uint4*>(&Vs[v_at(db * 16 + r, qg)]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < ATT_NT; ++j) lacc[j] = mfma16(ones4, pf0[j], lacc[j]);
@@ -583,7 +591,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
 #pragma unroll
             for (int i = 0; i < DH; ++i) {
                 const int db = (h == 0 ? DH : 0) + i;
-                if (db < D16) vf[i] = *reinterpret_cast<const uint4*>(&Vs[db * 16 + r][(h == 0 ? 0 : 32) + qg * 8]);
+                if (db < D16) vf[i] = *reinterpret_cast<const uint4*>(&Vs[v_at(db * 16 + r, (h == 0 ? 0 : 4) + qg)]);
             }
         }
 #pragma unroll
@@ -602,7 +610,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
 #pragma unroll
                 for (int i = 0; i < DH; ++i) {
                     const int db = DH + i;
-                    if (db < D16) vf[i] = *reinterpret_cast<const uint4*>(&Vs[db * 16 + r][32 + qg * 8]);
+                    if (db < D16) vf[i] = *reinterpret_cast<const uint4*>(&Vs[v_at(db * 16 + r, 4 + qg)]);
                 }
             }
         }
@@ -630,7 +638,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
                 for (int ks = 0; ks < KS; ++ks) {
                     const int dofs = ks * 32 + qg * 8;
                     kf[tau][ks] = (D % 32 == 0 || dofs < D)
-                                      ? *reinterpret_cast<const uint4*>(&Ks[row][D % 32 == 0 ? dofs : (dofs < D ? dofs : 0)])
+                                      ? *reinterpret_cast<const uint4*>(&Ks[k_at(row, (D % 32 == 0 ? dofs : (dofs < D ? dofs : 0)) / 8)])
                                       : zero4;
                 }
 #pragma unroll
@@ -711,7 +719,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
             const bool vok = key0 <= p_last && key0 + 8 > lo_first;   // else the tile holds another group's values
 #pragma unroll
             for (int db = 0; db < D16; ++db) {
-                const uint4 v = *reinterpret_cast<const uint4*>(&Vs[db * 16 + r][sub * 32 + qg * 8]);
+                const uint4 v = *reinterpret_cast<const uint4*>(&Vs[v_at(db * 16 + r, sub * 4 + qg)]);
                 const uint4 vf = (PAGE64 || vok) ? v : zero4;   // PAGE64: the tile's own page, finite, times p = 0
 #pragma unroll
                 for (int j = 0; j < ATT_NT; ++j) acc[j][db] = mfma16(vf, pf[j], acc[j][db]);
