@@ -82,6 +82,56 @@ def test_requests_that_share_a_beginning_share_its_pages(models, name):
     assert ran[False] - ran[True] == 32 + 24 + 32
 
 
+@pytest.mark.parametrize("name,dtype,graph,policy", [("A", "float32", False, "optimistic"), ("B", "bfloat16", True, "optimistic"),
+                                                     ("C", "bfloat16", True, "reserve_full")])
+def test_random_load_with_shared_beginnings_preemptions_and_graphs(models, name, dtype, graph, policy):
+    """Sixty requests that trickle in, with prompts cut from three stems, greedy and sampled, into a
+    pool of a few pages: after every step the cache manager's books agree; at the end everything
+    is finished and free, pages were shared, requests were preempted (optimistic admission), and in
+    float32 the greedy ones equal the plain implementation."""
+    import random
+    from infinilm_amd import LLM, SamplingParams
+
+    cfg, d, W = models[(name, dtype)]
+    V = cfg["vocab_size"]
+    rng = random.Random(5)
+    llm = LLM(d, dtype=dtype, num_blocks=12, block_size=8, max_batch_size=4, max_num_batched_tokens=64, chunk_size=16,
+              enable_graph=graph, admission=policy, seed=3)
+    eng = llm.engine
+    stems = [[rng.randrange(V) for _ in range(40)] for _ in range(3)]
+    reqs, pending, steps = [], 60, 0
+    while pending or eng.has_unfinished():
+        while pending and rng.random() < 0.3:
+            ids = rng.choice(stems)[:rng.randrange(1, 41)] + [rng.randrange(V) for _ in range(rng.randrange(0, 6))]
+            greedy = rng.random() < 0.6
+            sp = SamplingParams(top_k=1 if greedy else rng.choice([0, 5, 50]), top_p=1.0 if greedy else rng.choice([1.0, 0.9]),
+                                temperature=1.0 if greedy else rng.choice([0.7, 1.3]), max_tokens=rng.randrange(1, 30),
+                                ignore_eos=rng.random() < 0.5)
+            reqs.append((eng.add_request(ids, sp), ids, greedy))
+            pending -= 1
+        if eng.has_unfinished():
+            eng.step()
+            steps += 1
+            eng.runner.cache.check()
+        assert steps < 5000
+    assert all(r.is_finished() for r, _, _ in reqs)
+    assert all("no_capacity" in r.error for r, _, _ in reqs if r.error)
+    cache = eng.runner.cache
+    assert cache.free_pages() == 12 and not cache.requests
+    st = eng.stats()["cache"]
+    assert st["prefix_hit_tokens"] > 0
+    if policy == "optimistic":
+        assert st["preemptions"] > 0
+    if dtype == "float32":
+        checked = 0
+        for r, ids, greedy in reqs:
+            if greedy and not r.error and r.sampling_params.ignore_eos and checked < 6:
+                assert r.output_token_ids == P.plain_greedy(cfg, W, ids, r.sampling_params.max_tokens)
+                checked += 1
+        assert checked > 0
+    llm.close()
+
+
 def test_greedy_generation_bfloat16_with_graphs(models):
     """bfloat16 with decode steps replayed from captured graphs gives the same tokens as eager
     bfloat16 steps, and the plain implementation's up to near ties."""
