@@ -294,6 +294,17 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     # projection 22 -> 17 and 25 -> 19; up to 64 rows the library and a one-part sum are as fast)
     if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS:
         return _gemm_mid(a, w, K, False)
+    # 17 to 64 rows on their way into the residual sum: K in ranges of 1024 with the X fragments of all rows
+    # in registers (o projection at 64 rows 13.1 against the library's 18.9 us, down projection 33.9
+    # against 41.3, of which the sum of its 16 parts takes 5 back; up to 32 rows the down projection
+    # stays with the K-split kernel and its 4 parts)
+    if (fast and aligned and plain and allow_parts and out is None and 16 < M <= 64
+            and -(-K // ROWS64_SPAN) <= ROWS64_MAX_PARTS and (M > FEW_ROWS or K <= KSPLIT_SPAN)):
+        kb = -(-K // ROWS64_SPAN)
+        parts = torch.empty((kb, M, N), dtype=F32, device=a.device)
+        _run("ilm_gemm_rows64", parts.data_ptr(), N, M * N, kb, w.data_ptr(), w.stride(0), M, N, K, a.data_ptr(),
+             a.stride(0), _stream())
+        return parts
     if fast and aligned and plain and allow_parts and out is None and M <= max(16, FEW_ROWS) and K > KSPLIT_SPAN and USE_KSPLIT:
         kb = -(-K // KSPLIT_SPAN)
         parts = torch.empty((kb, M, N), dtype=F32, device=a.device)
@@ -338,6 +349,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     return out
 
 
+ROWS64_SPAN = 1024   # K range of one part of the 17-to-64-rows product (ilm_gemm_rows64_span())
+ROWS64_MAX_PARTS = int(os.environ.get("INFINILM_AMD_ROWS64_PARTS", "16"))   # 0: never this kernel
 MID_MAX_ROWS = int(os.environ.get("INFINILM_AMD_MID_ROWS", "128"))  # 16: above 16 rows always the library
 MID_TARGET_WGS = int(os.environ.get("INFINILM_AMD_MID_WGS", "512"))
 

@@ -38,6 +38,7 @@ def test_constants_mirrored_in_python_equal_the_library(K):
     assert L.ilm_attn_tile_tokens() == K.ATT_TILE_TOKENS
     assert L.ilm_attn_mfma_step() == K.ATT_STEP
     assert L.ilm_gemm_ksplit_max_k(1) == K.KSPLIT_SPAN
+    assert L.ilm_gemm_rows64_span() == K.ROWS64_SPAN
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -213,21 +214,22 @@ def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
     """Few rows and long K: the product comes as float32 parts; add_rmsnorm sums them in order."""
     a, w = _rand((M, K_), 14, torch.bfloat16), _rand((N, K_), 15, torch.bfloat16, 0.05)
     parts = K.gemm(a.to(DEV), w.to(DEV), allow_parts=True)
-    if 32 < M <= 64:   # the library serves these; the kernel itself is tested all the same
-        parts = K._gemm_mid(a.to(DEV), w.to(DEV), K_, False)
-    if parts.dim() == 2:   # short K: one float32 result
-        assert K_ <= 4096 and M <= 32
+    if 16 < M <= 64 and K_ % 8 == 0:   # K ranges of 1024 (up to 32 rows with K beyond 4096: ranges of 4096)
+        assert parts.shape[0] == (-(-K_ // 4096) if M <= 32 and K_ > 4096 else -(-K_ // 1024))
+        mid = K._gemm_mid(a.to(DEV), w.to(DEV), K_, False)   # not on this path, tested all the same
+        _close(mid.sum(0), P.plain_linear(a.to(F64), w.to(F64)), 1e-5)
+    if parts.dim() == 2:   # short K and few rows: one float32 result
+        assert K_ <= 4096 and M <= 16
         parts = parts[None]
     assert parts.dim() == 3 and parts.dtype == torch.float32
-    assert M > 32 or K_ <= 4096 or parts.shape[0] == -(-K_ // 4096)
+    assert M > 16 or K_ <= 4096 or parts.shape[0] == -(-K_ // 4096)
     want = P.plain_linear(a.to(F64), w.to(F64))
     _close(parts.sum(0), want, 1e-5)
     whole = K.gemm(a.to(DEV), w.to(DEV))
     assert whole.dim() == 2 and whole.dtype == torch.bfloat16
     short = K.gemm(a[:, :256].contiguous().to(DEV), w[:, :256].contiguous().to(DEV), allow_parts=True)
-    # short K: one part, not rounded to bfloat16 (more than 64 rows: the medium-rows kernel with its parts;
-    # 33 to 64: the library's bfloat16)
-    assert (short.dtype == torch.float32 and short.dim() == 2) if M <= 32 else (short.dim() == 3 if M > 64 else short.dtype == torch.bfloat16)
+    # short K: float32, not rounded to bfloat16 (more than 16 rows: parts)
+    assert (short.dtype == torch.float32 and short.dim() == 2) if M <= 16 else short.dim() == 3
     _close(whole, want, 6e-3)
     r = _rand((M, N), 16, scale=2.0)
     nw = _rand((N,), 17, torch.bfloat16) + 1
