@@ -93,12 +93,13 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __res
             v[it][4] = r1.x; v[it][5] = r1.y; v[it][6] = r1.z; v[it][7] = r1.w;
             if (h != nullptr) {
                 float hs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                // parts of a K-split product, summed in order; loaded four at a time, so that their
+                // parts of a K-split product, summed in order; loaded eight at a time, so that their
                 // latencies overlap (a product of many rows comes in up to 16 parts)
-                for (int p0 = 0; p0 < parts; p0 += 4) {
-                    HT hv[4][8];
+                constexpr int PB = 8;
+                for (int p0 = 0; p0 < parts; p0 += PB) {
+                    HT hv[PB][8];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
+                    for (int u = 0; u < PB; ++u) {
                         const int p = p0 + u < parts ? p0 + u : parts - 1;
                         const HT* hp = h + p * pstride + base + j;
                         if (sizeof(HT) == 2) {
@@ -109,7 +110,7 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __res
                         }
                     }
 #pragma unroll
-                    for (int u = 0; u < 4; ++u)
+                    for (int u = 0; u < PB; ++u)
                         if (p0 + u < parts) {
 #pragma unroll
                             for (int e = 0; e < 8; ++e) hs[e] += to_f32(hv[u][e]);
