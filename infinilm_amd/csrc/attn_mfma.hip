@@ -265,7 +265,16 @@ attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, cons
             const int dd = lane + 64 * i;
             if (dd < D) {
                 float a = o[i] * corr;
-                for (int j = 0; j < cnt; ++j) a += ws_acc[(base + g0 + j) * D + dd] * wsm[j];
+                const float* src = ws_acc + (base + g0) * D + dd;
+                int j = 0;
+                for (; j + 8 <= cnt; j += 8) {   // eight chunks' loads in flight; the sum keeps its order
+                    float v[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(j + u) * D];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) a += v[u] * wsm[j + u];
+                }
+                for (; j < cnt; ++j) a += src[(size_t)j * D] * wsm[j];
                 o[i] = a;
             }
         }
