@@ -7,7 +7,7 @@ A "step" is one decode step of the engine's own step function followed by greedy
 ends.  One JSON line is printed: `value` is decoded tokens a second at the default batch;
 `prefill` is one 2,048-token prompt in one step; `roofline` prices the decode step against HBM
 bandwidth (every weight it uses read once, plus the cache of the live requests); `points` holds
-decode at batch 1 and 64.  Peaks are MI355X's published ones (HBM 8 TB/s; dense MFMA bf16
+decode at batch 1, 32 and 64.  Peaks are MI355X's published ones (HBM 8 TB/s; dense MFMA bf16
 2.5 PFLOP/s, fp32 157.3 TFLOP/s).  Weights are random (N(0, 0.02), norms 1 + N(0, 0.02)) and the
 cache of the context is filled with random keys and values instead of being computed: the timed
 steps do all of their work.
@@ -57,7 +57,7 @@ def main() -> int:
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step eagerly")
     ap.add_argument("--prefill-only", action="store_true", help="only the prefill measurement (for profiling)")
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 32 / 64 points and the prefill")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (N>1 is not run)")
@@ -170,6 +170,7 @@ def main() -> int:
     if not args.no_points:
         k = max(8, args.steps // 2)
         record["points"] = {"decode_b1": round(decode(1, k, args.warmup)["tok_s"], 2),
+                            "decode_b32": round(decode(32, k, args.warmup)["tok_s"], 2),
                             "decode_b64": round(decode(64, k, args.warmup)["tok_s"], 2)}
         record["prefill"] = prefill()
     print(json.dumps(record))
