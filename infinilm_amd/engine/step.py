@@ -373,6 +373,49 @@ class StepRunner:
         except (CacheError, ValueError):
             self._prepared = None   # out of pages for the guess: the real step will say so if it comes
 
+    # ---- a decode step launched before the tokens of the one before it have come back -------------------
+    def ahead_ready(self, ids: Sequence) -> bool:
+        """The metadata of these requests' next decoded tokens lies prepared (their pages reserved)
+        and a graph for it is recorded: `step_ahead` can launch it without knowing the tokens."""
+        prep = self._prepared
+        if prep is None or not self.enable_graph:
+            return False
+        (key, pids, version), lengths, _ = prep
+        return (key in self._graphs and pids == tuple(ids) and version == self.cache.version
+                and lengths == [self.cache.length(i) for i in pids])
+
+    def step_ahead(self, ids: Sequence, tokens_dev: torch.Tensor) -> torch.Tensor:
+        """Launches the decode step whose input tokens are `tokens_dev` (int32 on the device, one a
+        request in the order of `ids`: what the sampler of the step before left there) and returns its
+        logits buffer.  The host has not seen the tokens: `commit_ahead` completes the step's books
+        once it has.  Needs `ahead_ready(ids)`."""
+        if not self.ahead_ready(ids):
+            raise RuntimeError("no prepared decode step for these requests")
+        prep, self._prepared = self._prepared, None
+        key = prep[0][0]
+        R = key[0]
+        graph, batch, logits, buf = self._graphs[key]
+        dev, host, turn, tok_off = prep[2]
+        if tokens_dev.dtype != torch.int32 or tokens_dev.numel() != R or tokens_dev.device != dev.device:
+            raise ValueError("the tokens of a step launched ahead are int32 on the device, one a request")
+        host.numpy()[tok_off:tok_off + R] = 0
+        self._copy_to_device(dev, host, turn)
+        dev[tok_off:tok_off + R].copy_(tokens_dev)    # behind the copy above on the stream
+        graph.replay()
+        self.steps += 1
+        self.tokens += R
+        return logits
+
+    def commit_ahead(self, id_tokens: Sequence) -> None:
+        """The books of a step launched by `step_ahead`, now that its input tokens are known:
+        (request, token) for every request that still exists (one that ended with the step before
+        is left out: what the step computed for it is never read).  Then the next step's metadata."""
+        live = [(i, t) for i, t in id_tokens if self.cache.has(i)]
+        for i, t in live:
+            self.cache.commit(i, 1, [t])
+        if live:
+            self._prepare_next_decode([StepEntry(i, [t], [0]) for i, t in live])
+
     def _graph_buffer_size(self, R: int, width: int) -> int:
         G = len(self.cache.groups)
         pad = lambda n: (n + 3) // 4 * 4

@@ -39,6 +39,8 @@ class LLM:
     temperature / top_p / top_k   defaults of requests that bring no SamplingParams
     max_num_batched_tokens / chunk_size   token budget of a step / longest portion of a prompt
     admission       "optimistic" (preempt when pages run out) | "reserve_full" (the reference's check)
+    look_ahead      with enable_graph: a decode step is launched before the tokens of the one before it are
+                    back on the host (None: on whenever enable_graph is)
     enable_prefix_caching   whole pages of computed tokens stay findable for later requests that begin
                     with the same tokens (the reference's default; off where a model's cache entries
                     keep a window or a state of their own)
@@ -50,7 +52,8 @@ class LLM:
                  enable_graph: bool = False, attn_backend: str = "default", skip_load: bool = False,
                  enable_prefix_caching: bool = True, max_num_batched_tokens: Optional[int] = None,
                  chunk_size: Optional[int] = None, admission: str = "optimistic", seed: int = 0,
-                 random_weights: bool = False, random_std: float = 0.02, tokenizer=None):
+                 random_weights: bool = False, random_std: float = 0.02, tokenizer=None,
+                 look_ahead: Optional[bool] = None):
         if cache_type != "paged":
             raise ValueError("only the paged cache exists here (cache_type='paged')")
         if attn_backend not in ("default", "paged-attn"):
@@ -78,7 +81,8 @@ class LLM:
         self.tokenizer = tokenizer
         self.enable_graph = enable_graph
         self.engine = LLMEngine(runner, max_num_seqs=max_batch_size, max_num_batched_tokens=max_num_batched_tokens,
-                                chunk_size=chunk_size, policy=admission, seed=seed, tokenizer=tokenizer)
+                                chunk_size=chunk_size, policy=admission, seed=seed, tokenizer=tokenizer,
+                                look_ahead=look_ahead)
 
     def _encode(self, prompt: str) -> List[int]:
         if self.tokenizer is None:

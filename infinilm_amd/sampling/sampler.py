@@ -37,24 +37,39 @@ def uniform_for(seed: int, request_key: int, index: int) -> float:
 class Sampler:
     def __init__(self, seed: int = 0):
         self.seed = int(seed)
-        self._staging = None    # pinned host memory for the rows' parameters
+        # pinned host memory for the rows' parameters: two buffers in turn, each waited for only when
+        # its own last copy may still be reading it (a step may be launched before the one before it
+        # has run)
+        self._staging = [None, None]
+        self._copied = [None, None]
+        self._turn = 0
 
     def sample(self, logits: torch.Tensor, rows: Sequence[Tuple[SamplingParams, int, int]]) -> List[int]:
         """`rows[i]` = (params, request key, index of the token being generated) for logits[i]."""
+        if logits.shape[0] == 0 and not rows:
+            return []
+        return self.sample_device(logits, rows).tolist()
+
+    def sample_device(self, logits: torch.Tensor, rows: Sequence[Tuple[SamplingParams, int, int]]) -> torch.Tensor:
+        """The same, the tokens left on the device (int32 [rows]); nothing waits for the stream."""
         n = logits.shape[0]
         if n != len(rows):
             raise ValueError(f"{n} rows of logits for {len(rows)} requests")
         if n == 0:
-            return []
+            raise ValueError("no rows to sample")
         if all(p.greedy for p, _, _ in rows):
-            return kernels.argmax(logits).tolist()
+            return kernels.argmax(logits)
         # temperature, top_k, top_p and the uniform numbers in one pinned buffer and one copy that
         # queues behind the step (a copy from pageable memory would make the host wait for the step
         # and the device wait for four copies)
         dev = logits.device
-        if self._staging is None or self._staging.numel() < 4 * n:
-            self._staging = torch.empty((4 * max(n, 64),), dtype=torch.float32, pin_memory=dev.type == "cuda")
-        host = self._staging[:4 * n]
+        t = self._turn = self._turn ^ 1
+        if self._copied[t] is not None:
+            self._copied[t].synchronize()
+            self._copied[t] = None
+        if self._staging[t] is None or self._staging[t].numel() < 4 * n:
+            self._staging[t] = torch.empty((4 * max(n, 64),), dtype=torch.float32, pin_memory=dev.type == "cuda")
+        host = self._staging[t][:4 * n]
         h = host.numpy()
         h[0:n] = [p.temperature for p, _, _ in rows]
         h[n:2 * n].view(np.int32)[:] = [p.top_k for p, _, _ in rows]
@@ -62,5 +77,7 @@ class Sampler:
         h[3 * n:4 * n] = [uniform_for(self.seed if p.seed is None else p.seed, key, idx) for p, key, idx in rows]
         d = torch.empty((4 * n,), dtype=torch.float32, device=dev)
         d.copy_(host, non_blocking=True)
-        tokens = kernels.sample(logits, d[0:n], d[n:2 * n].view(torch.int32), d[2 * n:3 * n], d[3 * n:4 * n])
-        return tokens.tolist()   # waits for the stream: the staging buffer is free again after this
+        if dev.type == "cuda":
+            self._copied[t] = torch.cuda.Event()
+            self._copied[t].record()
+        return kernels.sample(logits, d[0:n], d[n:2 * n].view(torch.int32), d[2 * n:3 * n], d[3 * n:4 * n])

@@ -132,6 +132,37 @@ def test_random_load_with_shared_beginnings_preemptions_and_graphs(models, name,
     llm.close()
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_decode_steps_launched_ahead_give_the_same_tokens(models, name):
+    """With recorded decode steps the engine launches a step before the tokens of the one before it
+    are back; the tokens fed on the device, the requests that end meanwhile (an end-of-sequence
+    token, a length) and the seeded sampling give what the step-by-step loop gives, token for token."""
+    from infinilm_amd import LLM, SamplingParams
+
+    cfg, d, W = models[(name, "bfloat16")]
+    V = cfg["vocab_size"]
+    prompts = [random_tokens(cfg, n, 700 + n) for n in (5, 21, 12, 40, 3, 17)]
+    ran = {}
+    for ahead in (False, True):
+        llm = LLM(d, dtype="float32", num_blocks=64, block_size=16, max_batch_size=4, enable_graph=True, look_ahead=ahead, seed=11)
+        eos = llm.engine.eos_token_ids
+        sps = [SamplingParams(top_k=1, max_tokens=30), SamplingParams(top_k=0, temperature=1.5, max_tokens=25),
+               SamplingParams(top_k=1, max_tokens=7, ignore_eos=True), SamplingParams(top_k=20, top_p=0.9, temperature=0.8, max_tokens=40),
+               SamplingParams(top_k=1, max_tokens=1), SamplingParams(top_k=0, temperature=2.0, max_tokens=33)]
+        # ends that no length foretells: every request stops at tokens that random sampling meets soon
+        for sp in sps[1::2]:
+            sp.stop_token_ids = list(range(0, V, 7))
+        outs = llm.generate(prompt_token_ids=prompts, sampling_params=sps)
+        ran[ahead] = [(o.outputs[0].token_ids, o.finish_reason) for o in outs]
+        st = llm.engine.stats()
+        assert (st["ahead_steps"] > 0) == ahead
+        assert llm.engine.runner.cache.free_pages() == 64
+        llm.engine.runner.cache.check()
+        llm.close()
+    assert ran[True] == ran[False]
+    assert any(r.value == "stop" for _, r in ran[True]), "no request ended on a stop token: the test does not test that"
+
+
 def test_greedy_generation_bfloat16_with_graphs(models):
     """bfloat16 with decode steps replayed from captured graphs gives the same tokens as eager
     bfloat16 steps, and the plain implementation's up to near ties."""
