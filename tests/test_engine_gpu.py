@@ -82,7 +82,7 @@ def test_requests_that_share_a_beginning_share_its_pages(models, name):
     assert ran[False] - ran[True] == 32 + 24 + 32
 
 
-@pytest.mark.parametrize("name,dtype,graph,policy", [("A", "float32", False, "optimistic"), ("B", "bfloat16", True, "optimistic"),
+@pytest.mark.parametrize("name,dtype,graph,policy", [("A", "float32", True, "optimistic"), ("B", "bfloat16", True, "optimistic"),
                                                      ("C", "bfloat16", True, "reserve_full")])
 def test_random_load_with_shared_beginnings_preemptions_and_graphs(models, name, dtype, graph, policy):
     """Sixty requests that trickle in, with prompts cut from three stems, greedy and sampled, into a
