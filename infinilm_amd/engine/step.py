@@ -297,14 +297,11 @@ class StepRunner:
     def _graph_key(self, entries: Sequence[StepEntry]):
         cache = self.cache
         need = max(-(-(cache.length(e.req_id) + 1) // cache.page_size) for e in entries)
-        width = 4
-        while width < need:
-            width *= 2
-        return (len(entries), width)
+        return (len(entries), kernels.bound_pages(need))
 
     def _graph_step(self, entries: Sequence[StepEntry], key) -> torch.Tensor:
-        """One graph per (number of requests, block-table width).  The width is rounded up to a power
-        of two, so a graph serves every context up to width * page tokens; the kernels' grids are
+        """One graph per (number of requests, block-table width).  The width is rounded up
+        (`kernels.bound_pages`: 4, 6, 8, 12, 16, ... pages), so a graph serves every context up to width * page tokens; the kernels' grids are
         sized for that bound and bound their reads by each request's own length.  Between replays
         only the metadata buffer changes (token ids, positions, slots, block tables).  A size is
         recorded the `graph_after`-th time it comes (a recording costs about three steps, which a

@@ -416,6 +416,16 @@ def swiglu_gemm(gate_up: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
 _NUM_CUS: dict = {}
 
 
+def bound_pages(need: int) -> int:
+    """The block-table width a context of `need` pages is served with: 4, 6, 8, 12, 16, 24, ... (at
+    most a third above the need).  The step function records one graph a width, and the attention
+    kernels size their grids for it, so an eager step and a replayed one cut their keys alike."""
+    width = 4
+    while width < need:
+        width = width * 3 // 2 if width & (width - 1) == 0 else width * 4 // 3
+    return width
+
+
 def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple:
     """(keys a chunk, chunks) of the chunked single-token attention for `pairs` = tokens x head groups.
 
@@ -426,11 +436,8 @@ def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple
     8 tokens 17.0 us with 256 keys a chunk (128: 18.4, 512: 20.2); 16 tokens 22.4 with 512 (256:
     24.0); 32 tokens 34.3 with 512 (256: 40.0, 1024: 36.5); 64 tokens 57.5 with 1024 (512: 60.5).
     At most ATT_MAX_CHUNKS chunks.  The length is first rounded up the way the step function rounds
-    its graphs' block tables (pages: 4, 8, 16, ...), so that an eager step and a replayed one cut alike."""
-    pages = 4
-    while pages * page < max_total_len:
-        pages *= 2
-    bound = pages * page
+    its graphs' block tables (`bound_pages`), so that an eager step and a replayed one cut alike."""
+    bound = bound_pages(-(-max_total_len // page)) * page
     cus = _NUM_CUS.get(device)
     if cus is None:
         cus = _NUM_CUS[device] = torch.cuda.get_device_properties(device).multi_processor_count
