@@ -1,4 +1,4 @@
-// Products with 17 to 128 rows of X (bfloat16) whose result goes into the residual sum: o and down
+// Products with 17 to 208 rows of X (bfloat16) whose result goes into the residual sum: o and down
 // projections of a decode step with many requests, or of a small portion of a prompt.  There the
 // vendor library leaves most of the chip idle (few output tiles, long K); here K is split over
 // blockIdx.y into float partial results C[y][M][N] that the next add+RMSNorm sums in order, so
@@ -43,7 +43,7 @@ __device__ __forceinline__ uint4 gm_swiglu8(uint4 g, uint4 up) {
     return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
-// MG: groups of 16 rows of X (2 .. 8); KT: k per step (128, or 64 where the X tiles would not fit)
+// MG: groups of 16 rows of X (2 .. 13); KT: k per step (128, or 64 where the X tiles would not fit)
 template <int MG, int KT, bool ACT>
 __global__ void __launch_bounds__(GM_THREADS)
 gemm_mid_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W, int M, int N, int K,
@@ -68,14 +68,20 @@ gemm_mid_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16* _
     // this thread's (at most two) pieces of an X tile: piece pc -> row pc / (KT/8), k offset (pc % (KT/8)) * 8.
     // Plain variables, not arrays: indexed arrays of registers end up in scratch memory here, and
     // every access to that waits for all loads in flight.
-    static_assert(XPER <= 2, "an X tile is at most two 16-byte pieces a thread");
-    const int pc0 = threadIdx.x, pc1 = threadIdx.x + GM_THREADS;
-    const int xk0 = pc0 % (KT / 8), xk1 = pc1 % (KT / 8);
+    static_assert(XPER <= 4, "an X tile is at most four 16-byte pieces a thread");
+    static_assert(sizeof(bf16) * 2 * MP * XROW <= 65536, "the two X tiles fit the LDS of a workgroup");
+    const int pc0 = threadIdx.x, pc1 = threadIdx.x + GM_THREADS, pc2 = threadIdx.x + 2 * GM_THREADS, pc3 = threadIdx.x + 3 * GM_THREADS;
+    const int xk0 = pc0 % (KT / 8), xk1 = pc1 % (KT / 8), xk2 = pc2 % (KT / 8), xk3 = pc3 % (KT / 8);
     const bool xok0 = pc0 < XPIECES && pc0 / (KT / 8) < M, xok1 = XPER > 1 && pc1 < XPIECES && pc1 / (KT / 8) < M;
+    const bool xok2 = XPER > 2 && pc2 < XPIECES && pc2 / (KT / 8) < M, xok3 = XPER > 3 && pc3 < XPIECES && pc3 / (KT / 8) < M;
     const uint4* xp0 = reinterpret_cast<const uint4*>(X + (size_t)(xok0 ? pc0 / (KT / 8) : 0) * lda);
     const uint4* xp1 = reinterpret_cast<const uint4*>(X + (size_t)(xok1 ? pc1 / (KT / 8) : 0) * lda);
+    const uint4* xp2 = reinterpret_cast<const uint4*>(X + (size_t)(xok2 ? pc2 / (KT / 8) : 0) * lda);
+    const uint4* xp3 = reinterpret_cast<const uint4*>(X + (size_t)(xok3 ? pc3 / (KT / 8) : 0) * lda);
     bf16* xs0 = &Xs[0][(pc0 < XPIECES ? pc0 : 0) / (KT / 8)][xk0 * 8];
     bf16* xs1 = &Xs[0][(pc1 < XPIECES ? pc1 : 0) / (KT / 8)][xk1 * 8];
+    bf16* xs2 = &Xs[0][(pc2 < XPIECES ? pc2 : 0) / (KT / 8)][xk2 * 8];
+    bf16* xs3 = &Xs[0][(pc3 < XPIECES ? pc3 : 0) / (KT / 8)][xk3 * 8];
     constexpr int XBUF = MP * XROW;   // elements between the two buffers
 #define GM_X_PIECE(DST_, XP_, XK_, OK_, STEP_)                                                     \
     {                                                                                              \
@@ -88,10 +94,14 @@ gemm_mid_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16* _
     }
 #define GM_LOAD_X(STEP_)                                                                           \
     GM_X_PIECE(x0, xp0, xk0, xok0, STEP_)                                                          \
-    if (XPER > 1) GM_X_PIECE(x1, xp1, xk1, xok1, STEP_)
+    if (XPER > 1) GM_X_PIECE(x1, xp1, xk1, xok1, STEP_)                                            \
+    if (XPER > 2) GM_X_PIECE(x2, xp2, xk2, xok2, STEP_)                                            \
+    if (XPER > 3) GM_X_PIECE(x3, xp3, xk3, xok3, STEP_)
 #define GM_STORE_X(BUF_)                                                                           \
     if (pc0 < XPIECES) *reinterpret_cast<uint4*>(xs0 + (BUF_) * XBUF) = x0;                        \
-    if (XPER > 1 && pc1 < XPIECES) *reinterpret_cast<uint4*>(xs1 + (BUF_) * XBUF) = x1;
+    if (XPER > 1 && pc1 < XPIECES) *reinterpret_cast<uint4*>(xs1 + (BUF_) * XBUF) = x1;        \
+    if (XPER > 2 && pc2 < XPIECES) *reinterpret_cast<uint4*>(xs2 + (BUF_) * XBUF) = x2;        \
+    if (XPER > 3 && pc3 < XPIECES) *reinterpret_cast<uint4*>(xs3 + (BUF_) * XBUF) = x3;
 #define GM_LOAD_W(DST_, STEP_)                                                                     \
     _Pragma("unroll") for (int s = 0; s < KSUB; ++s) {                                             \
         const int k8 = ((k_lo + (STEP_) * KT) >> 3) + s * 4 + q;                                   \
@@ -101,7 +111,7 @@ gemm_mid_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16* _
     f32x4 acc[MG];
 #pragma unroll
     for (int g = 0; g < MG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
-    uint4 x0 = zero, x1 = zero, wa[KSUB], wb[KSUB];
+    uint4 x0 = zero, x1 = zero, x2 = zero, x3 = zero, wa[KSUB], wb[KSUB];
     GM_LOAD_W(wa, 0)
     GM_LOAD_X(0)
     GM_STORE_X(0)
@@ -158,7 +168,7 @@ gemm_mid_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16* _
 // [y * kspan, (y + 1) * kspan), kspan a multiple of 128.  act != 0: X rows are [gate | up] (2K long).
 extern "C" int ilm_gemm_mid(void* C, int ldc, long c_part_stride, int kb, int kspan, const void* W, int ldw, int M, int N,
                             int K, const void* X, int lda, int act, hipStream_t stream) {
-    ILM_REQUIRE(M > 16 && M <= 128 && N > 0 && K > 0, "gemm_mid: needs 17 <= M <= 128, got M=%d N=%d K=%d", M, N, K);
+    ILM_REQUIRE(M > 16 && M <= 208 && N > 0 && K > 0, "gemm_mid: needs 17 <= M <= 208, got M=%d N=%d K=%d", M, N, K);
     ILM_REQUIRE(K % 8 == 0 && ldw % 8 == 0 && lda % 8 == 0 && ldw >= K && ldc >= N && lda >= (act ? 2 * K : K),
                 "gemm_mid: K=%d lda=%d ldw=%d ldc=%d", K, lda, ldw, ldc);
     ILM_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)C & 15) == 0 && (!act || K % 8 == 0),
@@ -178,7 +188,12 @@ extern "C" int ilm_gemm_mid(void* C, int ldc, long c_part_stride, int kb, int ks
         case 5: GM_LAUNCH(5); break;
         case 6: GM_LAUNCH(6); break;
         case 7: GM_LAUNCH(7); break;
-        default: GM_LAUNCH(8); break;
+        case 8: GM_LAUNCH(8); break;
+        case 9: GM_LAUNCH(9); break;
+        case 10: GM_LAUNCH(10); break;
+        case 11: GM_LAUNCH(11); break;
+        case 12: GM_LAUNCH(12); break;
+        default: GM_LAUNCH(13); break;
     }
 #undef GM_LAUNCH
     ILM_LAUNCH_CHECK("gemm_mid");
