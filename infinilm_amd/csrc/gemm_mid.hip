@@ -45,7 +45,7 @@ __device__ __forceinline__ uint4 gm_swiglu8(uint4 g, uint4 up) {
 
 // MG: groups of 16 rows of X (2 .. 13); KT: k per step (128, or 64 where the X tiles would not fit)
 template <int MG, int KT, bool ACT>
-__global__ void __launch_bounds__(GM_THREADS)
+__global__ void __launch_bounds__(GM_THREADS, 4)
 gemm_mid_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W, int M, int N, int K,
                 int lda, int ldw, int ldc, int kspan, size_t c_part_stride) {
     constexpr int MP = MG * 16;

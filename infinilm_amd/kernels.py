@@ -289,9 +289,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     aligned = K % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 \
         and w.data_ptr() % 16 == 0
     plain = bias is None and alpha == 1.0
-    # 65 to 192 rows on their way into the residual sum: split over K, where the vendor library leaves the
+    # 65 to 208 rows on their way into the residual sum: split over K, where the vendor library leaves the
     # chip idle (measured at the 8B shapes: down projection 68 -> 36 us at 96 rows, 81 -> 39 at 128, 92 -> 44
-    # at 160, 113 -> 68 at 192; o projection 22 -> 17 and 25 -> 19; at 208 rows the library is faster)
+    # at 160, 114 -> 48 at 192, 63 -> 51 at 208; o projection 22 -> 17, 25 -> 19, 32 -> 23 at 192)
     if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS:
         return _gemm_mid(a, w, K, False)
     # 17 to 64 rows on their way into the residual sum: K in ranges of 1024 with the X fragments of all rows
@@ -351,7 +351,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
 
 ROWS64_SPAN = 1024   # K range of one part of the 17-to-64-rows product (ilm_gemm_rows64_span())
 ROWS64_MAX_PARTS = int(os.environ.get("INFINILM_AMD_ROWS64_PARTS", "16"))   # 0: never this kernel
-MID_MAX_ROWS = int(os.environ.get("INFINILM_AMD_MID_ROWS", "192"))  # 16: above 16 rows always the library
+MID_MAX_ROWS = int(os.environ.get("INFINILM_AMD_MID_ROWS", "208"))  # 16: above 16 rows always the library
 MID_TARGET_WGS = int(os.environ.get("INFINILM_AMD_MID_WGS", "512"))
 
 

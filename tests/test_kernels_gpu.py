@@ -209,7 +209,7 @@ def test_gemm_bfloat16(K, M, N, K_, out_dtype):
 
 @pytest.mark.parametrize("M,N,K_", [(8, 4096, 16384), (1, 50, 8200), (16, 331, 12296), (17, 4096, 4096), (64, 4096, 16384),
                                     (48, 331, 200), (35, 50, 8200), (128, 1030, 1096), (97, 64, 72), (32, 4096, 16384),
-                                    (20, 331, 12296), (27, 50, 8200), (5, 96, 5760), (30, 2304, 5760), (192, 4096, 16384),
+                                    (20, 331, 12296), (27, 50, 8200), (5, 96, 5760), (30, 2304, 5760), (192, 4096, 16384), (208, 331, 4096),
                                     (150, 331, 1096), (177, 96, 200)])
 def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
     """Few rows and long K: the product comes as float32 parts; add_rmsnorm sums them in order."""
