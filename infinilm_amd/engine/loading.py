@@ -1,7 +1,7 @@
 """From a model folder to a built model with its weights, and to a step runner with a cache."""
 from __future__ import annotations
 
-from typing import Optional, Union
+from typing import Optional
 
 import torch
 

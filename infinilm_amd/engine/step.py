@@ -11,7 +11,7 @@ csrc/layers/attention/backends/paged_attn.cpp:36-37).
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np

@@ -8,7 +8,7 @@ prompts and single decoded tokens: a token at position p sees its request's keys
 """
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Dict
 
 import torch
 

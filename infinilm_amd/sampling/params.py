@@ -4,7 +4,7 @@ engine-level values for the whole batch (python/infinilm/llm/model_runner/model_
 each request's own temperature / top_p / top_k act, and `stop_token_ids` is honoured."""
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import List, Optional
 
 

@@ -17,7 +17,7 @@ from __future__ import annotations
 import glob
 import json
 import os
-from typing import Dict, Iterator, List, Tuple
+from typing import Iterator, List, Tuple
 
 import torch
 
