@@ -96,8 +96,10 @@ def main() -> int:
     greedy = SamplingParams(top_k=1)
     gen = torch.Generator().manual_seed(7)
 
-    layer_weight_bytes = sum(p.tensor.numel() * p.tensor.element_size() for n, p in model.named_parameters().items()
-                             if ".layers." in n or n.startswith(spec.final_norm_name))
+    # every tensor but the embedding table and the head: what the layers and the final norm read once a step
+    outer = {model.embed.data_ptr(), model.head.data_ptr()}
+    inner = [p.tensor for p in model.named_parameters().values() if p.tensor.data_ptr() not in outer]
+    layer_weight_bytes = sum(t.numel() * t.element_size() for t in inner)
     head_bytes = model.head.numel() * model.head.element_size()
 
     def decode(batch: int, steps: int, warmup: int):
@@ -146,8 +148,8 @@ def main() -> int:
             times.append(time.perf_counter() - t0)
             cache.release(rid)
         pt = min(times[1:])
-        mat_params = sum(p.tensor.numel() for n, p in model.named_parameters().items() if ".layers." in n and p.tensor.dim() == 2)
-        flops = 2.0 * T * mat_params + 4.0 * T * T / 2.0 * 32 * 128 * L + 2.0 * V * H
+        mat_params = sum(t.numel() for t in inner if t.dim() == 2)
+        flops = 2.0 * T * mat_params + 4.0 * T * T / 2.0 * cfg["num_attention_heads"] * cfg["head_dim"] * L + 2.0 * V * H
         return {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3), "frac": round(flops / pt / FLOP_PEAK[dkey], 4)}
 
     if args.prefill_only:

@@ -15,8 +15,9 @@ class BaseConfig:
         ap.add_argument("--model", type=str, required=True, help="model directory (config.json + safetensors)")
         ap.add_argument("--device", type=str, default="auto", help="always the AMD GPU; kept for compatibility")
         ap.add_argument("--device-id", type=int, default=0)
-        ap.add_argument("--dtype", type=str, default=None, choices=["float32", "bfloat16"],
-                        help="overrides config.json's dtype; float32 is true 32-bit throughout")
+        ap.add_argument("--dtype", type=str, default=None, choices=["float32", "bfloat16", "float16"],
+                        help="overrides config.json's dtype; float32 is true 32-bit throughout; float16 is run "
+                             "as bfloat16, with a warning")
         ap.add_argument("--batch-size", type=batch_size_type, default=batch_size_type(1),
                         help="number of copies of the prompt")
         ap.add_argument("--prompt", type=str, default="How are you")

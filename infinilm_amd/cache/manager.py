@@ -280,6 +280,19 @@ class CacheManager:
         r = self.requests[req_id]
         return (0 if r.fresh else r.state_slot), r.state_slot
 
+    def snapshot_states(self, req_ids: Sequence) -> list:
+        """Copies of the state rows these requests write, for `restore_states`: a step that has to run
+        twice on the same books (the warm-up before a graph is recorded) must not advance a state twice.
+        Keys and values need nothing of the kind: writing them again writes the same."""
+        if not self.state:
+            return []
+        rows = torch.tensor([self.requests[i].state_slot for i in req_ids], dtype=torch.long, device=self.device)
+        return [(pool, rows, pool.index_select(0, rows)) for pool in self.state.values()]
+
+    def restore_states(self, snapshot: list) -> None:
+        for pool, rows, saved in snapshot:
+            pool.index_copy_(0, rows, saved)
+
     def _publish(self, r: _Request, tokens: Sequence[int]) -> None:
         ps = self.page_size
         pool = self.groups[0].pool

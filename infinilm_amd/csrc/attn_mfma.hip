@@ -205,7 +205,7 @@ attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __re
         L += sm_ml[w][r][1] * wgt[w];
     }
     if (!head_ok) return;
-    const size_t slot = ((size_t)t * nh + head) * nsplit + split;
+    const size_t slot = ((size_t)blockIdx.x * nh + head) * nsplit + split;   // the workspace is laid out by served row
     for (int db = wave; db < D16; db += ATT_WAVES) {
         f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -242,7 +242,7 @@ attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, cons
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int s_lo = lo / span, s_hi = p / span;
-    const size_t base = ((size_t)t * nh + h) * nsplit;
+    const size_t base = ((size_t)blockIdx.x * nh + h) * nsplit;
     float o[4] = {0.f, 0.f, 0.f, 0.f};  // dims lane, lane+64, ... (D <= 256)
     float M = NEG_BIG, L = 0.f;
     // chunks in groups of 64: running rescale keeps one pass
@@ -688,7 +688,9 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
                     }
                 }
                 lm[j] = max3(max3(sv[j][0], sv[j][1], sv[j][2]), max3(sv[j][3], sv[j][4], sv[j][5]), max3(sv[j][6], sv[j][7], sv[j][7]));
-                over = over || fmaf(lm[j], scale_log2e, -mc[j]) > ATT_LAZY;
+                // (a column whose keys are all masked here leaves the reference point alone: it stays
+                // unset, which the mask-free path tests by its size)
+                over = over || (lm[j] > 0.5f * NEG_BIG && fmaf(lm[j], scale_log2e, -mc[j]) > ATT_LAZY);
             }
             if (__builtin_amdgcn_ballot_w64(over) != 0ull) {
 #pragma unroll
@@ -697,7 +699,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
                     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
                     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
                     const float mxc = mx * scale_log2e;
-                    const bool up = mxc - mc[j] > ATT_LAZY;   // the same in the four lanes of a column
+                    const bool up = mx > 0.5f * NEG_BIG && mxc - mc[j] > ATT_LAZY;   // the same in the four lanes of a column
                     const float corr = up ? __builtin_amdgcn_exp2f(mc[j] - mxc) : 1.0f;
                     mc[j] = up ? mxc : mc[j];
 #pragma unroll

@@ -21,7 +21,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libinfinilm_hip.so"
 ARCH = "gfx950"
 
-# (4) of the machine's traps: no packed-fp32 instructions from the compiler.
+# `-packed-fp32-ops` switched off: the compiler then makes no packed float32 instructions
+# (v_pk_add_f32, v_pk_mul_f32, v_pk_fma_f32) out of scalar or float2 code; some of their forms have
+# given wrong results on this hardware, now and then and without an error.
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -283,8 +283,9 @@ sample_reg_kernel(int* __restrict__ out, const float* __restrict__ logits, const
 #pragma unroll
     for (int e = EPT - 1; e >= 0; --e)
         if (keys[e] == kmax) first = threadIdx.x + e * NTH;
-    first = -(int)block_max_u<NW>((uint32_t)(-first), redu);   // min over the block (indices are >= 0)
-    if (first == 0x7fffffff || first < 0) first = 0;
+    // min over the block as a max of the complement (index 0 becomes the largest value)
+    first = 0x7fffffff - (int)block_max_u<NW>((uint32_t)(0x7fffffff - first), redu);
+    if (first == 0x7fffffff) first = 0;
     if (temp == 0.0f || k == 1) {
         if (threadIdx.x == 0) out[r] = first;
         return;

@@ -1,6 +1,7 @@
 """From a model folder to a built model with its weights, and to a step runner with a cache."""
 from __future__ import annotations
 
+import warnings
 from typing import Optional
 
 import torch
@@ -17,11 +18,18 @@ _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "fp32": torch.f
 
 def resolve_dtype(dtype, config_dtype: Optional[str]) -> torch.dtype:
     """`dtype` given wins; else config.json's `dtype`/`torch_dtype` (csrc/config/model_config.cpp:28-39).
-    float16 checkpoints run in bfloat16: the kernels here take float32 and bfloat16."""
+    float16 (a dtype of its own in the reference, csrc/utils.hpp:150-167) runs in bfloat16 here, with
+    a warning: the kernels take float32 and bfloat16, and bfloat16 keeps float16's range-safe
+    accumulation in float32 but three bits less of mantissa in weights, activations and cache."""
     if dtype is None:
         if config_dtype is None:
             raise ValueError("No dtype or torch_dtype found in config, and none was given")
-        dtype = "bfloat16" if config_dtype == "float16" else config_dtype
+        dtype = config_dtype
+    if dtype in ("float16", "fp16", "half", torch.float16):
+        warnings.warn("infinilm_amd: float16 was asked for; this engine computes in bfloat16 instead "
+                      "(same range as float32, 8 instead of 11 bits of precision): results differ from a "
+                      "float16 run by rounding. Pass dtype='float32' for the exact path.", RuntimeWarning, stacklevel=2)
+        dtype = "bfloat16"
     try:
         return _DTYPES[dtype]
     except KeyError:

@@ -111,6 +111,10 @@ class StepRunner:
         V = self.model.spec.vocab_size
         if not entries:
             raise ValueError("a step needs at least one entry")
+        if not defer_copy:
+            # prepared metadata lies in one of the two staging buffers that this step and the next take
+            # in turn: it does not outlive a step built in between
+            self._prepared = None
         seen = set()
         for e in entries:
             if e.req_id in seen:
@@ -315,7 +319,12 @@ class StepRunner:
             buf = torch.zeros((self._graph_buffer_size(R, width),), dtype=torch.int32, device=self.device)
             batch = self.build_batch(entries, min_blocks=width, device_buffer=buf)
             batch.max_total_len = width * cache.page_size     # grids are sized for the bound, not for this step
-            self.model.forward(batch, cache)                  # warm-up outside the capture; idempotent
+            # warm-up outside the capture (libraries set themselves up at their first call).  It runs the
+            # step that the first replay runs again: keys and values are written twice with the same
+            # values, fixed-size states are put back in between
+            saved = cache.snapshot_states([e.req_id for e in entries])
+            self.model.forward(batch, cache)
+            cache.restore_states(saved)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             if self._graph_pool is None:
@@ -339,7 +348,7 @@ class StepRunner:
                 self._copy_to_device(dev, host, turn)
             else:
                 fresh = self.build_batch(entries, min_blocks=width, device_buffer=buf)
-                if fresh.T != batch.T or fresh.block_tables[0].shape != batch.block_tables[0].shape:
+                if fresh.T != batch.T or [t.shape for t in fresh.block_tables] != [t.shape for t in batch.block_tables]:
                     raise RuntimeError("a decode step does not fit the graph captured for its size")
         graph.replay()
         for e in entries:

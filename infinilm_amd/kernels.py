@@ -499,8 +499,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         span, nsplit = attention_chunks(int(max_total_len), page, n_single * nkv * (-(-(nh // nkv) // 16)), q.device)
         ws_acc = ws_ml = None
         if nsplit > 1:
-            ws_acc = torch.empty((T * nh * nsplit * d,), dtype=F32, device=q.device)
-            ws_ml = torch.empty((T * nh * nsplit * 2,), dtype=F32, device=q.device)
+            # partial results of the rows served here (not of every token of the step)
+            ws_acc = torch.empty((n_single * nh * nsplit * d,), dtype=F32, device=q.device)
+            ws_ml = torch.empty((n_single * nh * nsplit * 2,), dtype=F32, device=q.device)
         _run("ilm_attn_mfma", out.data_ptr(), _ptr(ws_acc), _ptr(ws_ml), q.data_ptr(), k_cache.data_ptr(),
              v_cache.data_ptr(), block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), _ptr(rows),
              n_single, nh, nkv, d, page, block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window),

@@ -33,30 +33,28 @@ class GQAttention(Mixer):
                                ["q_proj", "k_proj", "v_proj"], qkv_bias, ctx)
         self.o_proj = Linear(self.nh * self.d, hidden_size, "o_proj", out_bias, ctx)
         self.position = build_position_encoding(position, ctx)
-        if self.position.rotary_dim > self.d:
-            raise ValueError("the position encoding rotates more dims than a head has")
+        if getattr(self.position, "head_dim", self.d) not in (0, self.d):
+            raise ValueError(f"the position encoding is made for heads of {self.position.head_dim}, the mixer's have {self.d}")
 
     def named_parameters(self) -> Dict[str, Param]:
         out = dict(self.qkv.named_parameters())
         out.update(self.o_proj.named_parameters())
+        for name, p in self.position.named_parameters().items():   # an encoding may bring tensors of its own
+            out[f"position.{name}"] = p
         return out
 
     def cache_need(self):
         return PagedKV(self.nkv, self.d, self.window)
 
     def forward(self, x: torch.Tensor, batch, cache_view) -> torch.Tensor:
-        if batch.max_position >= self.position.max_positions:
-            raise ValueError(f"position {batch.max_position} is beyond the position table ({self.position.max_positions})")
-        # few rows (decoded tokens): projection, rotation and cache write are one kernel
+        pe = self.position
+        pe.check(batch)
         qkv = None
-        if batch.taps is None and isinstance(self.position.cos, torch.Tensor):
-            qkv = kernels.qkv_rope_gemm(x, self.qkv.weight, self.qkv.bias, batch.positions, self.position.cos,
-                                        self.position.sin, cache_view.k, cache_view.v, cache_view.slots, self.nh,
-                                        self.nkv, self.d, self.position.rotary_dim)
+        if batch.taps is None:   # (a dump of the rotated rows needs them in one piece)
+            qkv = pe.project_encode_store(x, self.qkv, batch, cache_view, self.nh, self.nkv, self.d)
         if qkv is None:
             qkv = self.qkv.forward(x)
-            kernels.rope_kvwrite(qkv, batch.positions, self.position.cos, self.position.sin, cache_view.k, cache_view.v,
-                                 cache_view.slots, self.nh, self.nkv, self.d, self.position.rotary_dim)
+            pe.encode_and_store(qkv, batch, cache_view, self.nh, self.nkv, self.d)
             if batch.taps is not None:
                 batch.taps.setdefault("qkv_rotated", []).append(qkv.clone())
         o = kernels.paged_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,

@@ -11,7 +11,8 @@ which model it is in.
                                                    needs of the batch (segments, positions) and
                                                    of its cache view
   FeedForward      forward(x, batch)               x [T, hidden] -> [T, hidden]
-  PositionEncoding tables()/apply(x, positions)    consumed by mixers
+  PositionEncoding encode_and_store(qkv, batch, view, nh, nkv, d)   called by mixers: positions into
+                                                   q and k, encoded k and v into the cache
   Arrangement      forward(stream, batch, cache_view)  wires the slots around the residual stream
 """
 from __future__ import annotations
@@ -31,13 +32,16 @@ class BuildContext:
 class Param:
     """A named tensor of a part.  `tensor` is where the loader copies to (it may be a view into a
     fused buffer).  `keep_f32`: a tensor stored in 32-bit in the checkpoint stays 32-bit even when
-    the model runs in bfloat16 (the part's kernels take both)."""
+    the model runs in bfloat16 (the part's kernels take both).  `neutral`: the value at which the
+    tensor does nothing (1.0 for a norm's gain, 0.0 for matrices and biases); random weights may be
+    drawn around it."""
 
     def __init__(self, tensor: torch.Tensor, keep_f32: bool = False,
-                 replace: Optional[Callable[[torch.Tensor], None]] = None):
+                 replace: Optional[Callable[[torch.Tensor], None]] = None, neutral: float = 0.0):
         self.tensor = tensor
         self.keep_f32 = keep_f32 and replace is not None
         self._replace = replace
+        self.neutral = float(neutral)
 
     def replace(self, t: torch.Tensor) -> None:
         self._replace(t)
@@ -85,4 +89,32 @@ class FeedForward(Part):
 
 
 class PositionEncoding(Part):
-    pass
+    """How positions enter a mixer's queries and keys.  A mixer holds one, calls the three methods
+    below and never looks inside (tables, angles and kernels are the encoding's own), so another
+    encoding is a class of its own and no change to a mixer.
+
+      max_positions   positions from here on are refused (`check`)
+      encode_and_store(qkv, batch, view, nh, nkv, d)
+                      encodes `batch.positions` (or whatever of `batch` it reads) into the q and k heads
+                      of the fused projection rows qkv [T, (nh + 2 nkv) d], in place, and writes the
+                      encoded k and the v into the cache view (`view.k`, `view.v` at `view.slots`;
+                      nothing is written when `view.slots` is None).  The write belongs here because
+                      the kernel that touches k anyway does it in the same pass.
+      project_encode_store(x, proj, batch, view, nh, nkv, d) -> q or None
+                      optional short cut: projection, encoding and cache write in one kernel for the
+                      shapes an encoding has one for; returns the encoded queries [T, nh d], or None,
+                      after which the mixer runs `proj.forward(x)` and `encode_and_store`.
+    An encoding that cannot be written as a change of q and k (a bias on the scores) needs a mixer
+    that asks for it; the mixers here do not."""
+
+    max_positions: int = 1 << 30
+
+    def check(self, batch) -> None:
+        if batch.max_position >= self.max_positions:
+            raise ValueError(f"position {batch.max_position} is beyond the position encoding's {self.max_positions}")
+
+    def project_encode_store(self, x, proj, batch, view, nh: int, nkv: int, d: int):
+        return None
+
+    def encode_and_store(self, qkv, batch, view, nh: int, nkv: int, d: int) -> None:
+        raise NotImplementedError

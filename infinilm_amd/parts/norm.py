@@ -28,7 +28,7 @@ class RMSNorm(Norm):
         self.weight = t
 
     def named_parameters(self) -> Dict[str, Param]:
-        return {"weight": Param(self.weight, keep_f32=True, replace=self._set_weight)}
+        return {"weight": Param(self.weight, keep_f32=True, replace=self._set_weight, neutral=1.0)}
 
     def forward(self, stream: ResidualStream) -> torch.Tensor:
         x = kernels.add_rmsnorm(stream.residual, stream.pending, self.weight, stream.pending_scale, self.eps,

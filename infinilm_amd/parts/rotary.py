@@ -20,6 +20,7 @@ from typing import Callable, Dict, Optional, Tuple
 
 import torch
 
+from .. import kernels
 from .base import BuildContext, PositionEncoding
 from .registry import register_position_encoding
 
@@ -89,12 +90,24 @@ class RotaryEmbedding(PositionEncoding):
         ang = p[:, None] * inv_freq[None, :]
         return (torch.cos(ang) * m).to(torch.float32).contiguous(), (torch.sin(ang) * m).to(torch.float32).contiguous()
 
+    def project_encode_store(self, x, proj, batch, view, nh, nkv, d):
+        # few rows (decoded tokens): projection, rotation and cache write are one kernel
+        return kernels.qkv_rope_gemm(x, proj.weight, proj.bias, batch.positions, self.cos, self.sin, view.k, view.v,
+                                     view.slots, nh, nkv, d, self.rotary_dim)
+
+    def encode_and_store(self, qkv, batch, view, nh, nkv, d):
+        kernels.rope_kvwrite(qkv, batch.positions, self.cos, self.sin, view.k, view.v, view.slots, nh, nkv, d,
+                             self.rotary_dim)
+
 
 @register_position_encoding("none")
-class NoPositionEncoding(PositionEncoding):
-    """No rotation (rotary_dim 0)."""
+class NoPositionEncoding(RotaryEmbedding):
+    """No rotation (a rotary encoding over no dims): keys and values go to the cache as they are."""
 
     def __init__(self, ctx: BuildContext, head_dim: int = 0, **_):
         self.head_dim, self.rotary_dim, self.max_positions = int(head_dim), 0, 1 << 30
         self.cos = torch.zeros((1, 0), dtype=torch.float32, device=ctx.device)
         self.sin = torch.zeros((1, 0), dtype=torch.float32, device=ctx.device)
+
+    def project_encode_store(self, x, proj, batch, view, nh, nkv, d):
+        return None

@@ -4,8 +4,8 @@ seed, and an in-place fill of a built model on its device for runs too large to 
 The reference's `--skip-load` leaves device memory uninitialised
 (python/infinilm/llm/model_runner/model_runner.py:104-107); here weights are always drawn:
 every tensor N(0, std) from a generator seeded with (seed, position of the tensor in name order);
-`norm_init="one_plus"` draws 1-D norm weights as 1 + N(0, std) so that deep random models keep
-activations of order one.
+`norm_init="one_plus"` draws the tensors whose part declares a neutral value (`Param.neutral`: 1 for
+a norm's gain) as neutral + N(0, std), so that deep random models keep activations of order one.
 """
 from __future__ import annotations
 
@@ -38,8 +38,8 @@ def random_state_dict(config: dict, seed: int, std: float = 0.02, norm_init: str
             continue
         g = torch.Generator().manual_seed((int(seed) * 1000003 + i) & 0x7fffffffffff)
         t = torch.randn(tuple(p.tensor.shape), generator=g, dtype=torch.float32) * std
-        if norm_init == "one_plus" and t.dim() == 1 and "norm" in name:
-            t = t + 1.0
+        if norm_init == "one_plus" and p.neutral != 0.0:
+            t = t + p.neutral
         out[name] = t.to(store).contiguous()
     return out
 
@@ -81,5 +81,5 @@ def fill_random_(model, seed: int, std: float = 0.02, norm_init: str = "one_plus
             for a in range(0, flat.numel(), step):
                 b = min(flat.numel(), a + step)
                 flat[a:b] = (torch.randn((b - a,), generator=g, device=t.device, dtype=torch.float32) * std).to(t.dtype)
-        if norm_init == "one_plus" and t.dim() == 1 and "norm" in name:
-            t.add_(1.0)
+        if norm_init == "one_plus" and p.neutral != 0.0:
+            t.add_(p.neutral)

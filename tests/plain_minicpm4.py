@@ -158,9 +158,9 @@ def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: fl
     T, nh, d = q.shape
     nkv = k.shape[1]
     g = nh // nkv
-    rows = torch.arange(first_row, T)
+    rows = torch.arange(first_row, T, device=q.device)
     out = torch.empty_like(q[first_row:])
-    i = torch.arange(T)
+    i = torch.arange(T, device=q.device)
     mask = i[None, :] <= rows[:, None]
     if window > 0:
         mask &= i[None, :] > (rows[:, None] - window)
@@ -195,7 +195,7 @@ def plain_residual_scale(cfg: dict) -> float:
     return float(cfg.get("scale_depth", 1.0)) / math.sqrt(float(cfg["num_hidden_layers"]))
 
 
-def plain_self_attention(x, pos, cfg, W, prefix, cos, sin, alpha):
+def plain_self_attention(x, pos, cfg, W, prefix, cos, sin, alpha, taps=None):
     """qkv projection -> heads -> rotation of q and k -> attention -> o_proj * alpha.
 
     attention.cpp:96-137; slices in the order q, k, v: fused_linear.cpp:62-71; alpha on o_proj:
@@ -213,6 +213,10 @@ def plain_self_attention(x, pos, cfg, W, prefix, cos, sin, alpha):
     v = plain_linear(x, W[prefix + "v_proj.weight"], g("v_proj.bias")).view(T, nkv, d)
     q = plain_apply_rope(q, pos, cos, sin, rd)
     k = plain_apply_rope(k, pos, cos, sin, rd)
+    if taps is not None:
+        taps[prefix + "q_rotated"] = q.reshape(T, nh * d)
+        taps[prefix + "k_rotated"] = k.reshape(T, nkv * d)
+        taps[prefix + "v"] = v.reshape(T, nkv * d)
     o = plain_attention(q, k, v, 1.0 / math.sqrt(d)).reshape(T, nh * d)
     return plain_linear(o, W[prefix + "o_proj.weight"], g("o_proj.bias"), alpha)
 
@@ -229,23 +233,26 @@ def plain_forward(cfg: dict, weights: Dict[str, torch.Tensor], token_ids: Sequen
     final norm :99; head with alpha = dim_model_base / hidden_size only when the key exists
     :115-120; a checkpoint without lm_head.weight uses the unscaled embedding table:
     python/infinilm/modeling_utils.py:342-351.
-    `first_position` shifts all positions (used to test that only distances count).
+    `first_position` shifts all positions (used to test that only distances count).  `taps`
+    receives the residual stream after the embedding ("embed") and after every layer ("layer<l>"),
+    and each layer's rotated q, k and its v.  The computation runs where the weights lie.
     """
     W = {k: v.to(DT) for k, v in weights.items()}
-    ids = torch.as_tensor(list(token_ids), dtype=torch.long)
+    dev = W["model.embed_tokens.weight"].device
+    ids = torch.as_tensor(list(token_ids), dtype=torch.long, device=dev)
     T = ids.numel()
-    pos = torch.arange(T) + first_position
+    pos = torch.arange(T, device=dev) + first_position
     L = int(cfg["num_hidden_layers"])
     eps = float(cfg["rms_norm_eps"])
     alpha = plain_residual_scale(cfg)
-    cos, sin = plain_rope_tables(cfg)
+    cos, sin = (t.to(dev) for t in plain_rope_tables(cfg))
     x = plain_embedding(ids, W["model.embed_tokens.weight"], float(cfg.get("scale_emb", 1.0)))
     if taps is not None:
         taps["embed"] = x
     for l in range(L):
         p = f"model.layers.{l}."
         h = plain_rmsnorm(x, W[p + "input_layernorm.weight"], eps)
-        x = x + plain_self_attention(h, pos, cfg, W, p + "self_attn.", cos, sin, alpha)
+        x = x + plain_self_attention(h, pos, cfg, W, p + "self_attn.", cos, sin, alpha, taps)
         h = plain_rmsnorm(x, W[p + "post_attention_layernorm.weight"], eps)
         x = x + plain_mlp(h, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"],
                           W[p + "mlp.down_proj.weight"], alpha,

@@ -102,6 +102,14 @@ def test_state_slots():
     c.admit("c")
     assert c.state_rows("c") == (0, ra[1])
     c.check()
+    # a step that runs twice on the same books (the warm-up before a graph is recorded) puts the rows back
+    c.state[1][rb[1]] = 5.0
+    saved = c.snapshot_states(["b"])
+    c.state[1][rb[1]] += 1.0
+    c.state[1][ra[1]] = 9.0          # another request's row is not touched by the restore
+    c.restore_states(saved)
+    assert float(c.state[1][rb[1]].min()) == 5.0 == float(c.state[1][rb[1]].max()) and float(c.state[1][ra[1]].max()) == 9.0
+    assert _cache(needs=[PagedKV(1, 4)], max_requests=2).snapshot_states([]) == []
 
 
 @pytest.mark.parametrize("seed", range(6))

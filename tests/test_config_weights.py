@@ -209,3 +209,18 @@ def test_random_model_folder_roundtrip(tmp_path):
     assert ma.head_is_tied
     with pytest.raises(FileNotFoundError, match="Weight file not found"):
         load_weights(ma, str(tmp_path))
+
+
+def test_float16_is_run_as_bfloat16_with_a_warning():
+    """The reference has float16 as a dtype of its own (csrc/utils.hpp:150-167); this engine says
+    aloud that it computes such a model in bfloat16."""
+    import torch
+    from infinilm_amd.engine.loading import resolve_dtype
+
+    with pytest.warns(RuntimeWarning, match="bfloat16 instead"):
+        assert resolve_dtype(None, "float16") == torch.bfloat16
+    with pytest.warns(RuntimeWarning, match="bfloat16 instead"):
+        assert resolve_dtype("float16", "float32") == torch.bfloat16
+    assert resolve_dtype(None, "float32") == torch.float32
+    with pytest.raises(ValueError, match="Unsupported dtype"):
+        resolve_dtype("int8", None)

@@ -386,6 +386,28 @@ def test_attention_bfloat16_with_a_moving_maximum(K, ramp):
     _close(out, want, 1.2e-2)
 
 
+@pytest.mark.parametrize("d,page,window", [(128, 64, 128), (128, 64, 256), (64, 128, 192), (32, 256, 64)])
+def test_attention_bfloat16_window_edge_on_a_tile_boundary(K, d, page, window):
+    """A long portion under a window that is a multiple of the 64-key tile: one tile of tokens in
+    eight has its last token's window begin exactly where a key tile begins, so that token sees
+    nothing of the tile before (all its scores there are masked while it has seen no key yet) and
+    the next tile takes the mask-free path."""
+    out, want = _attention_case(K, torch.bfloat16, 4, 2, d, page, lens=[704, 333], qlens=[256, 200], window=window, seed=21)
+    _close(out, want, 1.2e-2)
+
+
+@pytest.mark.parametrize("nh,nkv,d,page", [(32, 2, 128, 256), (4, 2, 64, 128), (6, 3, 48, 256), (3, 1, 32, 128)])
+def test_attention_bfloat16_pages_longer_than_a_key_tile(K, nh, nkv, d, page):
+    """Pages of 128 and 256 keys: a 64-key tile begins in the middle of a page; portions with
+    history, decoded tokens beside them, a far key that dominates."""
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[700, 300, 65, 1], qlens=[100, 1, 65, 1], seed=31)
+    _close(out, want, 1.2e-2)
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[520, 900], qlens=[9, 1], seed=32, spike=True)
+    _close(out, want, 1.2e-2)
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=[600, 258], qlens=[77, 2], seed=33, window=130)
+    _close(out, want, 1.2e-2)
+
+
 @pytest.mark.parametrize("nh,nkv,d,page,n", [(8, 8, 64, 16, 40), (32, 2, 128, 64, 150), (4, 1, 32, 16, 120)])
 def test_attention_bfloat16_many_single_tokens(K, nh, nkv, d, page, n):
     """Many decoded tokens in one launch: the chunks get long (several 128-key steps a workgroup,
@@ -432,6 +454,11 @@ def test_argmax_and_sampling(K):
                         mk(u, torch.float32)).tolist()
 
     assert run(1.0, 1, 1.0, 0.5) == K.argmax(dl).tolist()           # top_k 1 is greedy
+    # a greedy row beside sampled rows, index 0 tied for the maximum: the first index wins there too
+    tie = logits.clone()
+    tie[0, 0] = tie[0, 5000] = tie[3, 0] = tie[3, V - 1] = 70.0
+    mixed = run([0.0, 1.0, 0.8, 1.0, 0.0], [0, 1, 40, 1, 0], 1.0, 0.3, tie)
+    assert mixed[0] == 0 and mixed[3] == 0 and mixed[1] == 100 and mixed[4] == int(torch.argmax(logits[4]))
     assert run(0.0, 0, 1.0, 0.9) == K.argmax(dl).tolist()           # temperature 0 is greedy
     # inverse CDF in vocabulary order against the plain implementation, over many u
     small = _rand((1, 331), 21, scale=2.0)

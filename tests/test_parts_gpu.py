@@ -190,6 +190,12 @@ def _register_toy():
 
         def forward(self, x, batch, view):
             u = x.float() @ self.wi.float().t()
+            if batch.all_decode:
+                # one token a request: rows by the device's index tensors, so that the step can be recorded
+                # as a graph and replayed for other requests (the host copies below would be baked in)
+                s = self.decay * view.pool.index_select(0, view.state_in.long()) + u
+                view.pool.index_copy_(0, view.state_out.long(), s)
+                return (s @ self.wo.float().t()).to(x.dtype)
             out = torch.empty_like(u)
             off = batch.h_seg_offsets
             for i in range(batch.R):
@@ -437,3 +443,163 @@ def test_toy_feed_forward_with_routing(tmp_path):
     drv.step([("a", a[19:])], end=["a"])
     assert rel_err(drv.request_logits("a", 45), plain(a)) < 1e-4
     assert rel_err(drv.request_logits("b", 20), plain(b)) < 1e-4
+
+
+def test_a_position_encoding_registered_from_outside(tmp_path):
+    """Another position encoding, defined here with a tensor of its own (a learned vector per
+    position added to every q and k head): registered, named in a layer, loaded by name and stepped in
+    portions and batches, without a change to the mixer or the step function."""
+    from safetensors.torch import save_file
+    from infinilm_amd import kernels
+    from infinilm_amd.config import HeadSpec, LayerRun, LayerSpec, ModelSpec, PartSpec, register_architecture
+    from infinilm_amd.engine.loading import build_model
+    from infinilm_amd.parts import Param, PositionEncoding, register_position_encoding
+    from helpers import Driver
+
+    @register_position_encoding("toy_learned_offsets")
+    class ToyLearnedOffsets(PositionEncoding):
+        def __init__(self, head_dim, max_positions, ctx):
+            self.head_dim, self.max_positions = int(head_dim), int(max_positions)
+            self.table = torch.empty((self.max_positions, self.head_dim), dtype=ctx.dtype, device=ctx.device)
+            self._none = torch.zeros((1, 0), dtype=torch.float32, device=ctx.device)
+
+        def named_parameters(self):
+            return {"offsets.weight": Param(self.table)}
+
+        def encode_and_store(self, qkv, batch, view, nh, nkv, d):
+            add = self.table[batch.positions.long()]                       # [T, d]
+            heads = qkv[:, :(nh + nkv) * d].view(-1, nh + nkv, d)           # q and k heads, not v
+            heads += add[:, None, :]
+            # the write alone: the rotation kernel over no dims
+            kernels.rope_kvwrite(qkv, batch.positions, self._none, self._none, view.k, view.v, view.slots, nh, nkv, d, 0)
+
+    H, d, nh, nkv, V, MAXP = 32, 16, 4, 2, 53, 96
+
+    def build_spec(cfg):
+        norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-6})
+        pos = PartSpec("toy_learned_offsets", {"head_dim": d, "max_positions": MAXP})
+        att = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d, "qkv_bias": False,
+                                         "out_bias": False, "scale": d ** -0.5, "window": 0, "position": pos})
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 40, "bias": False})
+        names = {"norm1": "ln1", "mixer": "att", "norm2": "ln2", "ffn": "ffn"}
+        layers = [LayerSpec(f"l.{i}", "pre_norm", {"norm1": norm, "mixer": att, "norm2": norm, "ffn": ffn}, names, 1.0) for i in range(2)]
+        return ModelSpec("ToyOffsetsLM", V, H, MAXP, "emb", 1.0, layers, [LayerRun(0, 0), LayerRun(1, 1)], norm, "ln_f",
+                         HeadSpec("head", 1.0, True))
+
+    register_architecture(["ToyOffsetsLM"], dict, build_spec)
+    cfg = {"architectures": ["ToyOffsetsLM"], "torch_dtype": "float32"}
+    mdir = str(tmp_path / "offsets")
+    os.makedirs(mdir)
+    json.dump(cfg, open(os.path.join(mdir, "config.json"), "w"))
+    names = build_model(cfg, "float32", "meta").named_parameters()
+    assert "l.1.att.position.offsets.weight" in names
+    g = torch.Generator().manual_seed(12)
+    W = {}
+    for name, p in sorted(names.items()):
+        if name == "head.weight":
+            continue
+        t = torch.randn(tuple(p.tensor.shape), generator=g) * 0.4
+        W[name] = (t * 0.25 + 1.0) if t.dim() == 1 else t
+    save_file(W, os.path.join(mdir, "model.safetensors"), metadata={"format": "pt"})
+
+    def plain(ids):
+        Wd = {k: v.to(F64) for k, v in W.items()}
+        n = len(ids)
+        x = Wd["emb.weight"][torch.tensor(ids)]
+        for l in range(2):
+            p = f"l.{l}."
+            h = P.plain_rmsnorm(x, Wd[p + "ln1.weight"], 1e-6)
+            off = Wd[p + "att.position.offsets.weight"][:n][:, None, :]
+            q = P.plain_linear(h, Wd[p + "att.q_proj.weight"]).view(n, nh, d) + off
+            k = P.plain_linear(h, Wd[p + "att.k_proj.weight"]).view(n, nkv, d) + off
+            v = P.plain_linear(h, Wd[p + "att.v_proj.weight"]).view(n, nkv, d)
+            x = x + P.plain_linear(P.plain_attention(q, k, v, d ** -0.5).reshape(n, nh * d), Wd[p + "att.o_proj.weight"])
+            h = P.plain_rmsnorm(x, Wd[p + "ln2.weight"], 1e-6)
+            x = x + P.plain_mlp(h, Wd[p + "ffn.gate_proj.weight"], Wd[p + "ffn.up_proj.weight"], Wd[p + "ffn.down_proj.weight"], 1.0)
+        return P.plain_linear(P.plain_rmsnorm(x, Wd["ln_f.weight"], 1e-6), Wd["emb.weight"])
+
+    drv = Driver(mdir, "float32", num_pages=16, page_size=8, max_requests=2)
+    g2 = torch.Generator().manual_seed(5)
+    a, b = (torch.randint(0, V, (n,), generator=g2).tolist() for n in (61, 18))
+    drv.step([("a", a[:30])])
+    drv.step([("a", a[30:32]), ("b", b)], end=["b"])
+    drv.step([("a", a[32:33])])
+    drv.step([("a", a[33:])], end=["a"])
+    assert rel_err(drv.request_logits("a", 61), plain(a)) < 1e-4
+    assert rel_err(drv.request_logits("b", 18), plain(b)) < 1e-4
+    with pytest.raises(ValueError, match="beyond the position encoding"):
+        drv.runner.cache.admit("c")
+        from infinilm_amd.engine.step import StepEntry
+        drv.runner.model.spec.max_positions = 1000   # the model's own bound lifted: the encoding's must hold
+        drv.runner.step([StepEntry("c", [1] * (MAXP + 1), [])])
+
+
+def test_a_model_without_paged_keys_runs_through_the_entry_point_with_graphs(tmp_path):
+    """Every mixer keeps a fixed-size state and none keeps pages: the scheduler's worst-case
+    admission, the recorded decode steps and the look-ahead loop have no block table to lean on."""
+    from safetensors.torch import save_file
+    from infinilm_amd import LLM, SamplingParams
+    from infinilm_amd.config import HeadSpec, LayerRun, LayerSpec, ModelSpec, PartSpec, register_architecture
+    from infinilm_amd.engine.loading import build_model
+
+    _register_toy()   # the toy mixer
+
+    def build_spec(cfg):
+        H = cfg["hidden_size"]
+        norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+        toy = PartSpec("toy_decay", {"hidden_size": H, "state_size": 20, "decay": 0.8})
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 48, "bias": False})
+        names = {"norm1": "ln1", "mixer": "mix", "norm2": "ln2", "ffn": "ffn"}
+        layers = [LayerSpec(f"b.{i}", "pre_norm", {"norm1": norm, "mixer": toy, "norm2": norm, "ffn": ffn}, names, 0.7) for i in range(2)]
+        return ModelSpec("ToyStateOnlyLM", cfg["vocab_size"], H, 512, "emb", 1.0, layers, [LayerRun(0, 0), LayerRun(1, 1)], norm,
+                         "ln_f", HeadSpec("head", 1.0, True))
+
+    register_architecture(["ToyStateOnlyLM"], dict, build_spec)
+    cfg = {"architectures": ["ToyStateOnlyLM"], "torch_dtype": "float32", "vocab_size": 71, "hidden_size": 32}
+    mdir = str(tmp_path / "state_only")
+    os.makedirs(mdir)
+    json.dump(cfg, open(os.path.join(mdir, "config.json"), "w"))
+    g = torch.Generator().manual_seed(2)
+    W = {}
+    for name, p in sorted(build_model(cfg, "float32", "meta").named_parameters().items()):
+        if name == "head.weight":
+            continue
+        t = torch.randn(tuple(p.tensor.shape), generator=g) * 0.4
+        W[name] = (t * 0.25 + 1.0) if t.dim() == 1 else t
+    save_file(W, os.path.join(mdir, "model.safetensors"), metadata={"format": "pt"})
+
+    def plain_logits(ids):
+        Wd = {k: v.to(F64) for k, v in W.items()}
+        x = Wd["emb.weight"][torch.tensor(ids)]
+        for l in range(2):
+            p = f"b.{l}."
+            h = P.plain_rmsnorm(x, Wd[p + "ln1.weight"], 1e-5)
+            u = h @ Wd[p + "mix.in_proj.weight"].T
+            s, rows = torch.zeros(20, dtype=F64), []
+            for t in range(len(ids)):
+                s = 0.8 * s + u[t]
+                rows.append(s)
+            x = x + 0.7 * (torch.stack(rows) @ Wd[p + "mix.out_proj.weight"].T)
+            h = P.plain_rmsnorm(x, Wd[p + "ln2.weight"], 1e-5)
+            x = x + 0.7 * P.plain_mlp(h, Wd[p + "ffn.gate_proj.weight"], Wd[p + "ffn.up_proj.weight"], Wd[p + "ffn.down_proj.weight"], 1.0)
+        return P.plain_linear(P.plain_rmsnorm(x, Wd["ln_f.weight"], 1e-5), Wd["emb.weight"])
+
+    def plain_greedy(ids, n):
+        ids, out = list(ids), []
+        for _ in range(n):
+            out.append(int(torch.argmax(plain_logits(ids)[-1])))
+            ids.append(out[-1])
+        return out
+
+    g2 = torch.Generator().manual_seed(6)
+    prompts = [torch.randint(0, 71, (n,), generator=g2).tolist() for n in (9, 1, 23, 14)]
+    for policy in ("reserve_full", "optimistic"):
+        llm = LLM(mdir, dtype="float32", num_blocks=4, block_size=16, max_batch_size=3, chunk_size=8, max_num_batched_tokens=16,
+                  enable_graph=True, admission=policy)
+        assert not llm.engine.runner.cache.groups
+        outs = llm.generate(prompt_token_ids=prompts, sampling_params=SamplingParams(top_k=1, max_tokens=12, ignore_eos=True))
+        for p, o in zip(prompts, outs):
+            assert o.outputs[0].token_ids == plain_greedy(p, 12), f"{policy}: prompt of {len(p)} tokens"
+        assert llm.engine.runner._graphs, "no decode step was recorded"
+        llm.engine.runner.cache.check()
+        llm.close()

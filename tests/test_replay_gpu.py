@@ -1,7 +1,10 @@
 """The engine against the plain implementation, through the engine's own step function: each
 request alone and whole; most of it in one step and the last 32 tokens one by one; in portions of
 changing size down to two tokens; and mixed, up to four live requests with so few pages that they
-are used again.  In 32-bit and in bfloat16, on tiny configurations that differ in every size."""
+are used again.  In 32-bit and in bfloat16, on tiny configurations that differ in every size, and
+over page sizes from 4 to 256 tokens: bfloat16 takes the matrix-core attention kernels from pages
+of 16 on (pages of 64 and more their one-lookup-a-tile path, pages of 256 a tile that begins in the
+middle of a page), the plain attention kernel below; 32-bit always the plain one."""
 import random
 
 import pytest
@@ -21,7 +24,7 @@ def case(request, tmp_path_factory):
     cfg = CONFIGS[name]()
     d = tmp_path_factory.mktemp(f"model_{name}_{dtype}")
     W = make_model_dir(str(d), cfg, seed=100 + ord(name), store=dtype)
-    n_max = min(cfg["max_position_embeddings"], 120)
+    n_max = min(cfg["max_position_embeddings"], 300)   # 128, 256 and 300 tokens: several pages of 64, key chunks of 128
     toks = {r: random_tokens(cfg, n, 7 * i + 1) for i, (r, n) in
             enumerate([("r0", n_max), ("r1", 1), ("r2", 45), ("r3", 70), ("r4", 2), ("r5", 97)])}
     oracle = {r: P.plain_forward(cfg, W, t) for r, t in toks.items()}
@@ -36,16 +39,52 @@ def _check(case, drv, rid):
     return err
 
 
-def test_each_request_alone_and_whole(case):
-    drv = Driver(case["dir"], case["dtype"], num_pages=64, page_size=16)
+def _pages(n_tokens, page):
+    return -(-n_tokens // page)
+
+
+class _KernelsSeen:
+    """Which attention kernels a test's steps launched (the library's own per-launch timers)."""
+
+    def __enter__(self):
+        from infinilm_amd import kernels
+        self.k = kernels
+        kernels.enable_timing(True)
+        return self
+
+    def __exit__(self, *exc):
+        self.calls = {name: rec["calls"] for name, rec in self.k.timing_report().items()}
+        self.k.enable_timing(False)
+        return False
+
+    def check(self, dtype, page, tile=True, single=True):
+        if dtype == "bfloat16" and page % 16 == 0:
+            assert "ilm_attn_basic" not in self.calls, "bfloat16 with pages of 16 and more must not take the plain attention"
+            assert not tile or self.calls.get("ilm_attn_tile", 0) > 0
+            assert not single or self.calls.get("ilm_attn_mfma", 0) > 0
+        else:
+            assert self.calls.get("ilm_attn_basic", 0) > 0
+
+
+@pytest.mark.parametrize("page", [16, 64, 256])
+def test_each_request_alone_and_whole(case, page):
+    num_pages = _pages(len(case["toks"]["r0"]), page) + 1
+    drv = Driver(case["dir"], case["dtype"], num_pages=num_pages, page_size=page)
     for rid, toks in case["toks"].items():
         drv.step([(rid, toks)], end=[rid])
         _check(case, drv, rid)
-    assert drv.runner.cache.free_pages() == 64
+    assert drv.runner.cache.free_pages() == num_pages
 
 
-def test_bulk_then_last_32_one_by_one(case):
-    drv = Driver(case["dir"], case["dtype"], num_pages=16, page_size=8)
+@pytest.mark.parametrize("page", [8, 16, 64, 256])
+def test_bulk_then_last_32_one_by_one(case, page):
+    drv = Driver(case["dir"], case["dtype"], num_pages=_pages(len(case["toks"]["r0"]), page) + 1, page_size=page)
+    with _KernelsSeen() as seen:
+        _bulk_then_last_32(case, drv)
+    seen.check(case["dtype"], page)
+
+
+def _bulk_then_last_32(case, drv):
     for rid in ("r0", "r3", "r5"):
         toks = case["toks"][rid]
         n = len(toks)
@@ -56,8 +95,15 @@ def test_bulk_then_last_32_one_by_one(case):
         drv.runner.cache.release(rid)
 
 
-def test_portions_of_changing_size(case):
-    drv = Driver(case["dir"], case["dtype"], num_pages=32, page_size=4)
+@pytest.mark.parametrize("page", [4, 16, 64, 256])
+def test_portions_of_changing_size(case, page):
+    drv = Driver(case["dir"], case["dtype"], num_pages=_pages(len(case["toks"]["r0"]), page) + 1, page_size=page)
+    with _KernelsSeen() as seen:
+        _portions_of_changing_size(case, drv)
+    seen.check(case["dtype"], page)
+
+
+def _portions_of_changing_size(case, drv):
     rng = random.Random(5)
     for rid in ("r0", "r2", "r3", "r5"):
         toks = case["toks"][rid]
@@ -75,10 +121,16 @@ def test_portions_of_changing_size(case):
         drv.runner.cache.release(rid)
 
 
-def test_mixed_batches_with_page_reuse(case):
+@pytest.mark.parametrize("page", [8, 16, 64, 256])
+def test_mixed_batches_with_page_reuse(case, page):
     """Up to four live requests; portions of some beside decoded tokens of others; the pool is so
     small that pages of finished requests are handed to new ones within the run."""
-    page = 8
+    with _KernelsSeen() as seen:
+        _mixed_batches_with_page_reuse(case, page)
+    seen.check(case["dtype"], page)
+
+
+def _mixed_batches_with_page_reuse(case, page):
     toks = case["toks"]
     order = ["r0", "r2", "r1", "r3", "r4", "r5", "r2b", "r0b"]
     toks = dict(toks, r2b=toks["r2"], r0b=toks["r0"])
@@ -92,7 +144,7 @@ def test_mixed_batches_with_page_reuse(case):
     waiting = list(order)
     live = {}          # rid -> tokens fed so far
     decode_from = {}   # rid -> position from which the request is fed one token a step
-    used_pages = set()
+    holders = {}       # page -> requests that have held it
     while waiting or live:
         while waiting and len(live) < 4:
             rid = waiting[0]
@@ -114,15 +166,21 @@ def test_mixed_batches_with_page_reuse(case):
                 ending.append(rid)
         if not entries:
             continue
-        drv.step(entries, end=ending)
+        drv.step(entries, end=[])
         for rid, _ in entries:
-            if rid not in ending:
-                used_pages.update(drv.runner.cache.table(rid, 0))
+            for pg in drv.runner.cache.table(rid, 0):
+                if pg >= 0:
+                    holders.setdefault(pg, set()).add(rid)
         for rid in ending:
+            drv.runner.cache.release(rid)
             del live[rid]
+        drv.runner.cache.check()
     for rid in order:
         err = rel_err(drv.request_logits(rid, len(toks[rid])), oracle[rid])
         print(f"[err] mixed {case['name']} {case['dtype']} {rid}: {err:.3e}")
         assert err < TOL[case["dtype"]], f"{case['name']} {case['dtype']} request {rid}: error {err:.3e}"
+    # pages went from finished requests to new ones (whose logits above are right although the pages
+    # were not cleared in between)
+    assert any(len(h) > 1 for h in holders.values()), "no page was held by two requests: the pool is not small enough"
     assert drv.runner.cache.free_pages() == num_pages
     drv.runner.cache.check()
