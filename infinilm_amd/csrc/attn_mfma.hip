@@ -23,6 +23,8 @@
 // Loads are unconditional 16-byte loads from clamped addresses, masked afterwards.
 // Needs: head size a multiple of 16 up to 128, page size a multiple of 16.
 #include "common.h"
+#include "no_alloc.h"
+#include <mutex>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -825,11 +827,11 @@ extern "C" int ilm_attn_tile(void* out, const void* q, const void* kc, const voi
 
 extern "C" int ilm_attn_mfma_step() { return ATT_STEP; }
 
-extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q, const void* kc,
-                             const void* vc, const void* block_tables, const void* seg, const void* pos,
-                             const void* rows, int T_, int nh, int nkv, int d, int page, int max_blocks,
-                             int q_stride, int out_stride, float scale, int window, int nsplit, int span,
-                             hipStream_t stream) {
+static int attn_mfma_launch(void* out, void* ws_acc, void* ws_ml, const void* q, const void* kc,
+                            const void* vc, const void* block_tables, const void* seg, const void* pos,
+                            const void* rows, int T_, int nh, int nkv, int d, int page, int max_blocks,
+                            int q_stride, int out_stride, float scale, int window, int nsplit, int span,
+                            hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_mfma: bad head counts nh=%d nkv=%d", nh, nkv);
     ILM_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attn_mfma: head size %d is not a multiple of 16 up to 128", d);
     ILM_REQUIRE(page % 16 == 0 && page > 0, "attn_mfma: page size %d is not a multiple of 16", page);
@@ -861,4 +863,68 @@ extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q
         ILM_LAUNCH_CHECK("attn_merge");
     }
     return 0;
+}
+
+extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q, const void* kc,
+                             const void* vc, const void* block_tables, const void* seg, const void* pos,
+                             const void* rows, int T_, int nh, int nkv, int d, int page, int max_blocks,
+                             int q_stride, int out_stride, float scale, int window, int nsplit, int span,
+                             hipStream_t stream) {
+    return attn_mfma_launch(out, ws_acc, ws_ml, q, kc, vc, block_tables, seg, pos, rows, T_, nh, nkv, d, page, max_blocks,
+                            q_stride, out_stride, scale, window, nsplit, span, stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same attention for callers that cannot allocate (see no_alloc.h): the chunks' partial results
+// go to a file-scope device array instead of a workspace the caller brings.
+// ------------------------------------------------------------------------------------------------
+static __device__ __align__(256) float scratch[ILM_ATTN_SCRATCH_FLOATS];
+
+// The array's device address, per device: each GPU holds its own copy at its own address.  In host
+// code the array's name is only a stand-in for the symbol; what kernels get is the pointer looked
+// up here, once per device, with that device current.
+#define ILM_MAX_DEVICES 64
+static float* scratch_ptr[ILM_MAX_DEVICES];
+static std::mutex scratch_mutex;
+
+static int scratch_of_current_device(float** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    ILM_REQUIRE(e == hipSuccess && dev >= 0 && dev < ILM_MAX_DEVICES, "attn_mfma_static: no current device (%s)",
+                hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_ptr[dev] == nullptr) {
+        float* p = nullptr;
+        e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        ILM_REQUIRE(e == hipSuccess && p != nullptr, "attn_mfma_static: the scratch array has no address on device %d (%s)",
+                    dev, hipGetErrorString(e));
+        scratch_ptr[dev] = p;
+    }
+    *ptr = scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" long ilm_attn_static_scratch_floats() { return (long)ILM_ATTN_SCRATCH_FLOATS; }
+
+extern "C" int ilm_attn_mfma_static(void* out, const void* q, const void* kc, const void* vc,
+                                    const void* block_tables, const void* seg, const void* pos, const void* rows,
+                                    int T_, int nh, int nkv, int d, int page, int max_blocks, int q_stride,
+                                    int out_stride, float scale, int window, int nsplit, int span,
+                                    hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && nh > 0 && d > 0 && nsplit >= 1, "attn_mfma_static: bad sizes T=%d nh=%d d=%d chunks=%d", T_, nh, d, nsplit);
+    float* ws_acc = nullptr;
+    float* ws_ml = nullptr;
+    if (nsplit > 1) {
+        const long long acc_floats = (long long)T_ * nh * nsplit * d, ml_floats = (long long)T_ * nh * nsplit * 2;
+        ILM_REQUIRE(acc_floats + ml_floats <= (long long)ILM_ATTN_SCRATCH_FLOATS,
+                    "attn_mfma_static: %d tokens x %d heads x %d chunks x (%d + 2) floats = %lld exceed the static "
+                    "scratch of %lld floats; use fewer chunks or tokens a call, or ilm_attn_mfma with a workspace",
+                    T_, nh, nsplit, d, acc_floats + ml_floats, (long long)ILM_ATTN_SCRATCH_FLOATS);
+        float* base = nullptr;
+        if (scratch_of_current_device(&base) != 0) return -1;
+        ws_acc = base;
+        ws_ml = base + acc_floats;   // d is a multiple of 16: 64-byte aligned
+    }
+    return attn_mfma_launch(out, ws_acc, ws_ml, q, kc, vc, block_tables, seg, pos, rows, T_, nh, nkv, d, page, max_blocks,
+                            q_stride, out_stride, scale, window, nsplit, span, stream);
 }

@@ -34,6 +34,7 @@ _SIGNATURES = {
     "ilm_attn_basic": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ilm_gemm_skinny": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ilm_attn_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+    "ilm_attn_mfma_static": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
     "ilm_attn_tile": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "ilm_argmax": [_P, _P, _I, _I, _I, _P],
     "ilm_sample": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
@@ -72,6 +73,8 @@ def load(verbose: bool = True) -> ctypes.CDLL:
                                "(python -c 'import __graft_entry__ as g; g.build()')")
         fn.argtypes = args
         fn.restype = c_int
+    lib.ilm_attn_static_scratch_floats.restype = c_long
+    lib.ilm_attn_static_scratch_floats.argtypes = []
     _lib = lib
     return lib
 
