@@ -29,19 +29,9 @@ FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 def config_8b(layers: int) -> dict:
     """The layer sizes of the MiniCPM4-8B shape."""
-    import torch
-    g = torch.Generator().manual_seed(1234)
-    short = (1.0 + 3.0 * torch.rand(64, generator=g)).tolist()
-    long = (1.0 + 3.0 * torch.rand(64, generator=g)).tolist()
-    return {
-        "architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm", "torch_dtype": "bfloat16",
-        "num_hidden_layers": layers, "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 2,
-        "head_dim": 128, "intermediate_size": 16384, "vocab_size": 73448, "rope_theta": 10000.0,
-        "max_position_embeddings": 32768, "rms_norm_eps": 1e-6, "scale_emb": 12, "scale_depth": 1.4,
-        "dim_model_base": 256, "tie_word_embeddings": False,
-        "rope_scaling": {"type": "longrope", "short_factor": short, "long_factor": long,
-                         "original_max_position_embeddings": 32768},
-    }
+    sys.path.insert(0, os.path.join(ROOT, "examples"))
+    from shapes import shape_config
+    return shape_config("8b", layers)
 
 
 def main() -> int:
