@@ -370,15 +370,21 @@ def _gemm_mid(x: torch.Tensor, w: torch.Tensor, K: int, act: bool) -> torch.Tens
 
 
 USE_GATEUP_SWIGLU = os.environ.get("INFINILM_AMD_GATEUP_SWIGLU", "1") == "1"
+USE_GATEUP_WIDE = os.environ.get("INFINILM_AMD_GATEUP_WIDE", "1") == "1"
 
 
 def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
     """silu(x Wg^T + bg) * (x Wu^T + bu) for few rows in bfloat16, W = [Wg; Wu]: the fused gate/up
-    projection with the SwiGLU in its epilogue, [M, I].  None where the kernel does not apply (too many
-    rows, float32, K beyond the registers): the caller then runs the projection and the activation."""
+    projection with the SwiGLU in its epilogue, [M, I] (up to 32 rows with X in registers, up to 64 with X
+    through LDS).  None where no kernel applies (more rows, float32): the caller then runs the projection
+    and the activation."""
     M, K = x.shape
+    resident = _few_rows(M, K) and K <= 8192
+    # 17 to 64 rows that do not fit the registers: X through LDS, W streamed over the whole K by every wave
+    # (64 rows at the 8B shape: 52 us against 62 + 5 for the vendor library's product and the activation kernel)
+    wide = USE_GATEUP_WIDE and not resident and 16 < M <= 64
     if not (USE_GATEUP_SWIGLU and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and x.is_cuda
-            and _few_rows(M, K) and K <= 8192 and K % 8 == 0 and w.shape[0] % 2 == 0 and w.shape[1] == K
+            and (resident or wide) and K % 8 == 0 and w.shape[0] % 2 == 0 and w.shape[1] == K
             and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         return None
@@ -387,8 +393,8 @@ def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
     if bias is not None and (bias.shape != (2 * I,) or bias.dtype != BF16 or not bias.is_contiguous()):
         raise KernelError("bias does not fit the fused gate/up projection")
     out = torch.empty((M, I), dtype=BF16, device=x.device)
-    _run("ilm_gemm_gateup_swiglu", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
-         _ptr(bias), M, I, K, _stream())
+    _run("ilm_gemm_gateup_swiglu" if resident else "ilm_gemm_gateup_wide", out.data_ptr(), out.stride(0), x.data_ptr(),
+         x.stride(0), w.data_ptr(), w.stride(0), _ptr(bias), M, I, K, _stream())
     return out
 
 

@@ -261,7 +261,10 @@ def test_swiglu_inside_the_down_projection(K, M, I, N):
 
 @pytest.mark.parametrize("M,I,Kd,bias", [(8, 16384, 4096, False), (3, 200, 96, True), (16, 331, 1032, False), (17, 331, 1032, True),
                                          (32, 4096, 4096, False), (5, 50, 8192, True), (24, 96, 200, False),
-                                         (20, 8200, 1032, True), (2, 5760, 2304, False)])
+                                         (20, 8200, 1032, True), (2, 5760, 2304, False),
+                                         # 33 to 64 rows, and 17 to 32 with a long K: X through LDS
+                                         (64, 16384, 4096, False), (33, 331, 1032, True), (48, 200, 96, False), (49, 4100, 520, True),
+                                         (40, 5760, 2304, False), (64, 61, 8, True), (20, 96, 8200, False)])
 def test_gate_up_projection_with_the_activation_in_its_epilogue(K, M, I, Kd, bias):
     """One kernel for silu(x Wg^T) * (x Wu^T) against the plain formula and against the projection
     followed by the activation kernel (gate and up rounded to bfloat16 at the same place)."""
@@ -276,7 +279,7 @@ def test_gate_up_projection_with_the_activation_in_its_epilogue(K, M, I, Kd, bia
     assert (act.float() - two.float()).abs().max() <= 2 ** -6 * max(float(two.float().abs().max()), 1e-6)
     assert K.gateup_swiglu_gemm(dev(x.float()), dev(w.float()), None) is None          # float32: not this kernel
     if M <= 32:
-        big = _rand((33, Kd), 34, torch.bfloat16)
+        big = _rand((65, Kd), 34, torch.bfloat16)
         assert K.gateup_swiglu_gemm(dev(big), dev(w), dev(b)) is None                  # too many rows
 
 
