@@ -40,6 +40,20 @@ extern "C" int ilm_embed(void* r, const void* ids, const void* table, int T_, in
     return 0;
 }
 
+// eight consecutive elements as floats (16-byte accesses; p must be 16-byte aligned)
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float* v) {
+    T t[8];
+    if (sizeof(T) == 2) {
+        *reinterpret_cast<uint4*>(t) = *reinterpret_cast<const uint4*>(p);
+    } else {
+        *reinterpret_cast<float4*>(t) = *reinterpret_cast<const float4*>(p);
+        *reinterpret_cast<float4*>(t + 4) = *reinterpret_cast<const float4*>(p + 4);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = to_f32(t[e]);
+}
+
 // ------------------------------------------------------------------------------------------
 // r += alpha * h ; x = r / sqrt(mean(r^2) + eps) * w
 // One block per row.  The sum of squares is reduced in an order that depends on H only, so a
@@ -125,6 +139,13 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __res
             for (int e = 0; e < 8; ++e) ss += v[it][e] * v[it][e];
         }
     }
+    // the weights are on their way while the sum of squares is reduced
+    float wv[NITER][8];
+#pragma unroll
+    for (int it = 0; it < NITER; ++it) {
+        const int j = (it * 256 + threadIdx.x) * 8;
+        load8<WT>(w + (j < H ? j : 0), wv[it]);
+    }
     const float tot = block_sum<4>(ss, red);
     const float rstd = 1.0f / sqrtf(tot / (float)H + eps);
 #pragma unroll
@@ -133,7 +154,7 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __res
         if (j < H) {
             T o[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = from_f32<T>(v[it][e] * rstd * to_f32(w[j + e]));
+            for (int e = 0; e < 8; ++e) o[e] = from_f32<T>(v[it][e] * rstd * wv[it][e]);
             if (sizeof(T) == 2) {
                 *reinterpret_cast<uint4*>(x + base + j) = *reinterpret_cast<uint4*>(o);
             } else {
@@ -154,7 +175,7 @@ extern "C" int ilm_add_rmsnorm(void* x, void* r, const void* h, const void* w, i
                 "add_rmsnorm: the branch must have the activations' dtype or be float, in >= 1 parts");
     // H a multiple of 8 up to 8192 with 16-byte aligned rows takes the vector kernel
     const bool vec = H % 8 == 0 && H <= 8192 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)r & 15) == 0 &&
-                     ((uintptr_t)h & 15) == 0 && pstride % 8 == 0;
+                     ((uintptr_t)h & 15) == 0 && ((uintptr_t)w & 15) == 0 && pstride % 8 == 0;
     const int niter = (H + 2047) / 2048;
     const bool hf = h != nullptr && h_dtype == ILM_DTYPE_F32;
 #define NORM_LAUNCH(T, WT, HT)                                                                                   \
@@ -235,18 +256,6 @@ rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ pos, const floa
 
 // Vector form: one block a token, every thread 8 consecutive dims of a pair (16-byte accesses).
 // Needs rd a multiple of 16 (half the rotary dims in steps of 8) and d a multiple of 8.
-template <typename T>
-__device__ __forceinline__ void load8(const T* p, float* v) {
-    T t[8];
-    if (sizeof(T) == 2) {
-        *reinterpret_cast<uint4*>(t) = *reinterpret_cast<const uint4*>(p);
-    } else {
-        *reinterpret_cast<float4*>(t) = *reinterpret_cast<const float4*>(p);
-        *reinterpret_cast<float4*>(t + 4) = *reinterpret_cast<const float4*>(p + 4);
-    }
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = to_f32(t[e]);
-}
 template <typename T>
 __device__ __forceinline__ void store8(T* p, const T* t) {
     if (sizeof(T) == 2) {

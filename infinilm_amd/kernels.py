@@ -20,6 +20,9 @@ _DT = {torch.float32: 0, torch.bfloat16: 1}
 ATT_TILE_TOKENS = 8  # tokens per tile of the prompt-portion attention kernel (ilm_attn_tile_tokens())
 ATT_STEP = 128  # keys a workgroup of the chunked attention takes in one step (ilm_attn_mfma_step())
 ATT_MAX_CHUNKS = 64  # most chunks a context is cut into (the merge kernel walks them one after the other)
+BASIC_CHUNK = 512    # keys a chunk of the plain attention kernel (ilm_attn_basic_chunk())
+BASIC_SPLIT = os.environ.get("INFINILM_AMD_BASIC_SPLIT", "1") == "1"   # 0: always one wave a (token, head)
+BASIC_SPLIT_WAVES = 4096   # (token, head) pairs up to which the plain kernel takes one wave a chunk
 # INFINILM_AMD_BASIC=1 runs the plain kernels everywhere (for telling a kernel's fault from the engine's)
 FORCE_BASIC = os.environ.get("INFINILM_AMD_BASIC", "0") == "1"
 SKINNY_VARIANT = int(os.environ.get("INFINILM_AMD_SKINNY_VARIANT", "0"))  # 0: the kernel chooses
@@ -344,9 +347,20 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
         with _timed("library_gemm"):
             torch.matmul(a, w.t(), out=out)
         return out
+    if (a.dtype == F32 and out_dtype == F32 and not FORCE_BASIC and M <= F32_FEW_ROWS and K % 4 == 0 and a.stride(0) % 4 == 0
+            and w.stride(0) % 4 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        # the 32-bit path's few rows (decoded tokens): W streamed once on the float matrix instruction
+        _run("ilm_gemm_f32_skinny", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
+             w.stride(0), out.stride(0), float(alpha), _stream())
+        return out
     _run("ilm_gemm_basic", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0), w.stride(0),
          out.stride(0), float(alpha), _dt(a), _DT[out_dtype], _stream())
     return out
+
+
+# Rows up to which the 32-bit products take the few-rows kernel (0: always the ascending-k kernel, whose sums
+# do not depend on the number of rows at all)
+F32_FEW_ROWS = int(os.environ.get("INFINILM_AMD_F32_FEW_ROWS", "64"))
 
 
 ROWS64_SPAN = 1024   # K range of one part of the 17-to-64-rows product (ilm_gemm_rows64_span())
@@ -513,8 +527,15 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
              n_single, nh, nkv, d, page, block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window),
              nsplit, span, _stream())
         return out
-    _run("ilm_attn_basic", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
-         seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d, page, block_tables.shape[1],
+    # The plain kernel.  Few tokens over long contexts (decoding): one wave a chunk of keys and a fold of the
+    # partial results, instead of one wave a head; the bits are the same (see attn_basic.hip).
+    ws, nchunks = None, 1
+    bound = block_tables.shape[1] * page if max_total_len is None else int(max_total_len)
+    if BASIC_SPLIT and T * nh <= BASIC_SPLIT_WAVES and bound > BASIC_CHUNK:
+        nchunks = -(-bound // BASIC_CHUNK)
+        ws = torch.empty((T * nh * nchunks * (d + 2),), dtype=F32, device=q.device)
+    _run("ilm_attn_basic", out.data_ptr(), _ptr(ws), nchunks, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+         block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d, page, block_tables.shape[1],
          q.stride(0), out.stride(0), float(scale), int(window), _dt(q), _stream())
     return out
 

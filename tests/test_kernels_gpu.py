@@ -37,6 +37,7 @@ def test_constants_mirrored_in_python_equal_the_library(K):
     L = lib.load()
     assert L.ilm_attn_tile_tokens() == K.ATT_TILE_TOKENS
     assert L.ilm_attn_mfma_step() == K.ATT_STEP
+    assert L.ilm_attn_basic_chunk() == K.BASIC_CHUNK
     assert L.ilm_gemm_ksplit_max_k(1) == K.KSPLIT_SPAN
     assert L.ilm_gemm_rows64_span() == K.ROWS64_SPAN
 
@@ -175,15 +176,25 @@ def test_swiglu_and_gather(K, dtype):
     assert torch.equal(K.gather_rows(x.to(DEV), idx.to(DEV)).cpu(), x[idx.long()])
 
 
-@pytest.mark.parametrize("M,N,K_", [(1, 1, 1), (5, 331, 80), (64, 96, 200), (130, 70, 33), (3, 4608, 4096)])
+@pytest.mark.parametrize("M,N,K_", [(1, 1, 1), (5, 331, 80), (64, 96, 200), (130, 70, 33), (3, 4608, 4096), (17, 331, 4100),
+                                    (33, 50, 12296), (48, 4608, 1032), (8, 16400, 64), (20, 32768, 256), (200, 96, 200)])
 def test_gemm_float32_is_true_float32(K, M, N, K_):
     a, w, b = _rand((M, K_), 8), _rand((N, K_), 9), _rand((N,), 10)
     out = K.gemm(a.to(DEV), w.to(DEV), b.to(DEV), 0.25)
     want = P.plain_linear(a.to(F64), w.to(F64), b.to(F64), 0.25)
     _close(out, want, 2e-6 * math.sqrt(K_))   # no reduced-precision matrix mode: errors of float32 sums only
-    # rows do not depend on the batch around them, bit for bit
+    # Rows do not depend on the batch around them, bit for bit, among calls of up to 64 rows (the few-rows
+    # kernel) and among calls of more (the ascending-k kernel); between the two, by the rounding of a
+    # float32 sum in another order.
     one = K.gemm(a[M // 2:M // 2 + 1].to(DEV), w.to(DEV), b.to(DEV), 0.25)
-    assert torch.equal(one.cpu(), out[M // 2:M // 2 + 1].cpu())
+    if M <= 64:
+        assert torch.equal(one.cpu(), out[M // 2:M // 2 + 1].cpu())
+        some = K.gemm(a[:min(M, 3)].to(DEV), w.to(DEV), b.to(DEV), 0.25)
+        assert torch.equal(some.cpu(), out[:min(M, 3)].cpu())
+    else:
+        _close(one, out[M // 2:M // 2 + 1], 1e-6 * math.sqrt(K_))
+        more = K.gemm(torch.cat([a, a[:70]]).to(DEV), w.to(DEV), b.to(DEV), 0.25)
+        assert torch.equal(more[:M].cpu(), out.cpu())
 
 
 @pytest.mark.parametrize("M,N,K_,out_dtype", [
@@ -360,6 +371,20 @@ def test_attention_float32(K, nh, nkv, d, page):
     _close(out, want, 3e-6)
     out, want = _attention_case(K, torch.float32, nh, nkv, d, page, lens=[300, 65], qlens=[1, 1], seed=9, spike=True)
     _close(out, want, 3e-6)
+
+
+def test_attention_float32_one_wave_a_chunk_gives_the_same_bits(K, monkeypatch):
+    """The plain kernel's two launch shapes (one wave walks all chunks of a token and head; one wave a
+    chunk and a fold) agree bit for bit, so that a token decoded alone and the same token inside a
+    portion of a prompt cannot differ."""
+    case = dict(lens=[1500, 700, 513, 40], qlens=[1, 1, 3, 1])
+    for window in (0, 600):
+        monkeypatch.setattr(K, "BASIC_SPLIT", True)
+        split, want = _attention_case(K, torch.float32, 6, 2, 48, 8, window=window, seed=4, **case)
+        monkeypatch.setattr(K, "BASIC_SPLIT", False)
+        whole, _ = _attention_case(K, torch.float32, 6, 2, 48, 8, window=window, seed=4, **case)
+        assert torch.equal(split.cpu(), whole.cpu())
+        _close(split, want, 3e-6)
 
 
 @pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 16), (3, 1, 32, 16), (6, 3, 48, 32), (32, 2, 128, 64), (16, 16, 64, 16),
