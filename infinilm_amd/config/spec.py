@@ -40,9 +40,13 @@ class LayerRun:
 
 @dataclass
 class HeadSpec:
+    """The output head: a part of kind `kind` built from (vocab_size, hidden_size, scale, **params), whose
+    tensors lie under `name` in a checkpoint."""
     name: str = "lm_head"
     scale: float = 1.0
     tie_to_embedding_when_missing: bool = True
+    kind: str = "linear"
+    params: Dict[str, Any] = field(default_factory=dict)
 
 
 @dataclass
@@ -59,6 +63,9 @@ class ModelSpec:
     final_norm_name: str
     head: HeadSpec
     eos_token_ids: List[int] = field(default_factory=list)
+    # the embedding: a part of kind `embed_kind` built from (vocab_size, hidden_size, scale=embed_scale, **embed_params)
+    embed_kind: str = "scaled_lookup"
+    embed_params: Dict[str, Any] = field(default_factory=dict)
 
     def num_cache_entries(self) -> int:
         ids = [r.cache for r in self.order if r.cache is not None]

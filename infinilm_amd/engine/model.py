@@ -1,5 +1,6 @@
 """The generic causal language model: embedding, layers run in the order the description gives,
-final norm, output head at the wanted rows.  It is built from a `ModelSpec` alone.
+final norm, output head at the wanted rows.  It is built from a `ModelSpec` alone; the embedding and
+the head are parts chosen by kind like the layers' (`parts/ends.py`).
 
 Reference for the flow: csrc/models/minicpm4/minicpm4_for_causal_lm.cpp:89-101 (model loop),
 :123-127 (head); gathering the wanted rows before the head follows the generic template
@@ -13,9 +14,9 @@ from typing import Dict, List, Optional
 import torch
 
 from .. import kernels
-from ..config.spec import ModelSpec
+from ..config.spec import ModelSpec, PartSpec
 from ..parts import BuildContext, Param, ResidualStream, build_block
-from ..parts.registry import build_norm
+from ..parts.registry import build_embedding, build_head, build_norm
 
 
 class CausalLM:
@@ -25,12 +26,12 @@ class CausalLM:
         self.dtype = dtype
         self.device = torch.device(device)
         ctx = BuildContext(dtype=dtype, device=self.device)
-        self.embed = torch.empty((spec.vocab_size, spec.hidden_size), dtype=dtype, device=self.device)
+        self.embedding = build_embedding(PartSpec(spec.embed_kind, dict(spec.embed_params, vocab_size=spec.vocab_size,
+                                                                         hidden_size=spec.hidden_size, scale=spec.embed_scale)), ctx)
         self.blocks = [build_block(ls, ctx) for ls in spec.layers]
         self.final_norm = build_norm(spec.final_norm, ctx)
-        self.head: Optional[torch.Tensor] = torch.empty((spec.vocab_size, spec.hidden_size), dtype=dtype,
-                                                        device=self.device)
-        self.head_is_tied = False
+        self.output_head = build_head(PartSpec(spec.head.kind, dict(spec.head.params, vocab_size=spec.vocab_size,
+                                                                    hidden_size=spec.hidden_size, scale=spec.head.scale)), ctx)
         # cache entry -> what its writer's mixer needs
         self.cache_needs: List = [None] * spec.num_cache_entries()
         for run in spec.order:
@@ -44,27 +45,37 @@ class CausalLM:
                                      f"{self.cache_needs[run.cache]}, but needs {need}")
 
     # ---- tensors by checkpoint name ---------------------------------------------------------
-    def _set_embed(self, t):
-        self.embed = t
+    @property
+    def embed(self) -> torch.Tensor:
+        """The embedding's table."""
+        return self.embedding.table
 
-    def _set_head(self, t):
-        self.head = t
+    @property
+    def head(self) -> torch.Tensor:
+        """The head's matrix (the embedding's table itself when the head is tied)."""
+        return self.output_head.weight
+
+    @property
+    def head_is_tied(self) -> bool:
+        return self.output_head.tied
 
     def named_parameters(self) -> Dict[str, Param]:
-        out: Dict[str, Param] = {f"{self.spec.embed_name}.weight": Param(self.embed)}
+        out: Dict[str, Param] = {}
+        for name, p in self.embedding.named_parameters().items():
+            out[f"{self.spec.embed_name}.{name}"] = p
         for b in self.blocks:
             out.update(b.named_parameters())
         for name, p in self.final_norm.named_parameters().items():
             out[f"{self.spec.final_norm_name}.{name}"] = p
-        out[f"{self.spec.head.name}.weight"] = Param(self.head)
+        for name, p in self.output_head.named_parameters().items():
+            out[f"{self.spec.head.name}.{name}"] = p
         return out
 
     def tie_head_to_embedding(self) -> None:
         """The head reads the embedding table itself (one tensor, no copy); the embedding's scale
         is applied at lookup, so the table the head sees is the unscaled one
         (python/infinilm/modeling_utils.py:342-351)."""
-        self.head = self.embed
-        self.head_is_tied = True
+        self.output_head.tie(self.embedding.table)
 
     def weight_bytes(self) -> int:
         seen = {}
@@ -76,7 +87,7 @@ class CausalLM:
     # ---- forward ------------------------------------------------------------------------------
     def forward(self, batch, cache) -> torch.Tensor:
         """float32 logits [len(batch.want_rows), vocab] for the tokens of `batch`."""
-        stream = ResidualStream(kernels.embed(batch.token_ids, self.embed, self.spec.embed_scale))
+        stream = ResidualStream(self.embedding.forward(batch.token_ids))
         taps = batch.taps
         if taps is not None:
             taps["embed"] = stream.residual.clone()
@@ -99,4 +110,4 @@ class CausalLM:
                 last.push(pend, stream.pending_scale)
             stream = last
         x = self.final_norm.forward(stream)
-        return kernels.gemm(x, self.head, None, self.spec.head.scale, torch.float32)
+        return self.output_head.forward(x)

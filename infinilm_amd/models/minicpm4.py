@@ -49,6 +49,7 @@ class RopeScaling:
     long_factor: Optional[List[float]] = None
     original_max_position_embeddings: Optional[int] = None
     factor: float = 1.0
+    extra: Optional[dict] = None   # the other keys of a kind (llama3: low/high_freq_factor; yarn: beta_*, mscale*)
 
 
 @dataclass
@@ -168,6 +169,23 @@ class MiniCPM4Config:
             raise ConfigError("rope_scaling must contain 'type' or 'rope_type' field")
         if kind in ("default", "none", "dynamic"):
             return None
+        if kind == "llama3":   # rope_scaling_creators.cpp:54-75
+            need = ("factor", "low_freq_factor", "high_freq_factor", "original_max_position_embeddings")
+            if any(k not in rs for k in need):
+                raise ConfigError("Llama3RopeScalingConfig requires 'factor', 'low_freq_factor', 'high_freq_factor', and "
+                                  "'original_max_position_embeddings'")
+            if float(rs["high_freq_factor"]) <= float(rs["low_freq_factor"]) or float(rs["factor"]) <= 0:
+                raise ConfigError("llama3 rope scaling needs factor > 0 and high_freq_factor > low_freq_factor")
+            return RopeScaling("llama3", None, None, int(rs["original_max_position_embeddings"]), float(rs["factor"]),
+                               {"low_freq_factor": float(rs["low_freq_factor"]), "high_freq_factor": float(rs["high_freq_factor"])})
+        if kind == "yarn":     # rope_scaling_creators.cpp:80-102 (keys and their defaults)
+            if "factor" not in rs or "original_max_position_embeddings" not in rs:
+                raise ConfigError("YarnRopeScalingConfig requires 'factor' and 'original_max_position_embeddings'")
+            if float(rs["factor"]) <= 0:
+                raise ConfigError("yarn rope scaling needs factor > 0")
+            return RopeScaling("yarn", None, None, int(rs["original_max_position_embeddings"]), float(rs["factor"]),
+                               {"beta_fast": int(float(rs.get("beta_fast", 32.0))), "beta_slow": int(float(rs.get("beta_slow", 1.0))),
+                                "mscale": float(rs.get("mscale", 1.0)), "mscale_all_dim": float(rs.get("mscale_all_dim", 0.0))})
         if kind != "longrope":
             raise ConfigError(f"Unsupported rope_scaling_type: {kind}")
         for k in ("short_factor", "long_factor", "original_max_position_embeddings"):
@@ -193,8 +211,10 @@ def build_spec(cfg: MiniCPM4Config) -> ModelSpec:
     scaling = None
     if cfg.rope_scaling is not None:
         s = cfg.rope_scaling
-        scaling = {"type": s.kind, "short_factor": s.short_factor, "long_factor": s.long_factor,
-                   "original_max_position_embeddings": s.original_max_position_embeddings, "factor": s.factor}
+        scaling = {"type": s.kind, "original_max_position_embeddings": s.original_max_position_embeddings, "factor": s.factor}
+        if s.kind == "longrope":
+            scaling.update(short_factor=s.short_factor, long_factor=s.long_factor)
+        scaling.update(s.extra or {})
     position = PartSpec("rotary", {"head_dim": cfg.head_dim, "rotary_dim": cfg.rotary_dim,
                                    "max_positions": cfg.max_position_embeddings, "theta": cfg.rope_theta,
                                    "scaling": scaling})

@@ -3,7 +3,7 @@
 Reference: csrc/layers/rotary_embedding/rotary_embedding.cpp:90-113 (one table for
 max_position_embeddings positions, shared by the layers), rotary_embedding_factory.cpp:11-39 (kind
 from `type` or `rope_type`; absent/null = none), rope_scaling_creators.cpp:23-47,106-115 (longrope's
-keys; `default`, `none`, `dynamic` = no scaling), csrc/config/model_config.hpp:139 (rotate-half
+keys; `default`, `none`, `dynamic` = no scaling; `llama3` and `yarn` below), csrc/config/model_config.hpp:139 (rotate-half
 pairing).  The arithmetic is the tensor library's in the reference; the definition used:
 
   inv_freq_i = 1 / (f_i * theta^(2i/rd)),  i < rd/2
@@ -56,6 +56,46 @@ def _longrope(inv_freq, params, max_positions):
     return inv_freq / f, m
 
 
+@register_rope_scaling("llama3")
+def _llama3(inv_freq, params, max_positions, theta=None):
+    """Keys: rope_scaling_creators.cpp:54-75 (factor, low_freq_factor, high_freq_factor,
+    original_max_position_embeddings).  The arithmetic is in the reference's tensor library, not in its
+    text (parity unpinned); the definition used, with wavelength 2 pi / inv_freq and o the original length:
+      wavelength < o / high_freq_factor  ->  unchanged
+      wavelength > o / low_freq_factor   ->  inv_freq / factor
+      between: s = (o / wavelength - low_freq_factor) / (high_freq_factor - low_freq_factor),
+               inv_freq * ((1 - s) / factor + s)."""
+    factor, lo, hi = float(params["factor"]), float(params["low_freq_factor"]), float(params["high_freq_factor"])
+    orig = float(params["original_max_position_embeddings"])
+    wavelen = 2.0 * math.pi / inv_freq
+    s = ((orig / wavelen - lo) / (hi - lo)).clamp(0.0, 1.0)   # 0 below the low band's edge, 1 above the high one's
+    return inv_freq * ((1.0 - s) / factor + s), 1.0
+
+
+@register_rope_scaling("yarn")
+def _yarn(inv_freq, params, max_positions, theta=None):
+    """Keys and defaults: rope_scaling_creators.cpp:80-102 (factor, original_max_position_embeddings,
+    beta_fast 32, beta_slow 1, mscale 1, mscale_all_dim 0; rotary dim and rope_theta from the model).
+    The arithmetic is in the reference's tensor library, not in its text (parity unpinned); the
+    definition used, with D the rotary dim, b = theta and o the original length:
+      c(beta) = D ln(o / (2 pi beta)) / (2 ln b)            the pair index that turns beta times within o
+      lo = max(floor(c(beta_fast)), 0), hi = min(ceil(c(beta_slow)), D/2 - 1)
+      ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)   0: turns often, kept; 1: turns seldom, stretched
+      inv_freq_i * (1 - ramp_i) + inv_freq_i / factor * ramp_i
+      magnitude = g(mscale) / g(mscale_all_dim), g(m) = 0.1 m ln(factor) + 1 for factor > 1, else 1."""
+    factor, orig = float(params["factor"]), float(params["original_max_position_embeddings"])
+    half = inv_freq.numel()
+    D = 2 * half
+    base = float(theta if theta is not None else params.get("rope_theta", 10000.0))
+    corr = lambda beta: D * math.log(orig / (2.0 * math.pi * beta)) / (2.0 * math.log(base))
+    lo = max(math.floor(corr(float(params.get("beta_fast", 32)))), 0)
+    hi = min(math.ceil(corr(float(params.get("beta_slow", 1)))), half - 1)
+    i = torch.arange(half, dtype=torch.float64)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    g = lambda m: 0.1 * m * math.log(factor) + 1.0 if factor > 1.0 else 1.0
+    return inv_freq * (1.0 - ramp) + inv_freq / factor * ramp, g(float(params.get("mscale", 1.0))) / g(float(params.get("mscale_all_dim", 0.0)))
+
+
 _TABLE_CACHE: Dict[Tuple, Tuple[torch.Tensor, torch.Tensor]] = {}
 
 
@@ -85,7 +125,12 @@ class RotaryEmbedding(PositionEncoding):
             kind = self.scaling.get("type", self.scaling.get("rope_type"))
             if kind not in SCALINGS:
                 raise ValueError(f"Unsupported rope_scaling_type: {kind}")
-            inv_freq, m = SCALINGS[kind](inv_freq, self.scaling, self.max_positions)
+            fn = SCALINGS[kind]
+            # a scaling that takes a fourth argument is given the base theta (yarn's band edges need it)
+            if fn.__code__.co_argcount >= 4:
+                inv_freq, m = fn(inv_freq, self.scaling, self.max_positions, self.theta)
+            else:
+                inv_freq, m = fn(inv_freq, self.scaling, self.max_positions)
         p = torch.arange(self.max_positions, dtype=torch.float64)
         ang = p[:, None] * inv_freq[None, :]
         return (torch.cos(ang) * m).to(torch.float32).contiguous(), (torch.sin(ang) * m).to(torch.float32).contiguous()

@@ -224,3 +224,44 @@ def test_float16_is_run_as_bfloat16_with_a_warning():
     assert resolve_dtype(None, "float32") == torch.float32
     with pytest.raises(ValueError, match="Unsupported dtype"):
         resolve_dtype("int8", None)
+
+
+def test_llama3_and_yarn_rope_scalings_are_accepted_with_their_keys():
+    """The other two kinds the reference's factory knows (rope_scaling_creators.cpp:54-102): keys,
+    defaults and error messages as there; the arithmetic is not in the reference's text (parity
+    unpinned), so it is pinned here by what the definitions imply: frequencies that turn often stay,
+    those that turn seldom are divided by the factor, in between they change monotonically."""
+    from infinilm_amd.parts.rotary import SCALINGS
+
+    base = P.tiny_config_a()
+    for rs, msg in [({"type": "llama3", "factor": 8.0}, "Llama3RopeScalingConfig requires"),
+                    ({"rope_type": "yarn", "factor": 4.0}, "YarnRopeScalingConfig requires")]:
+        with pytest.raises(ConfigError, match=msg):
+            load_model_config(dict(base, rope_scaling=rs))
+    _, cfg = load_model_config(dict(base, rope_scaling={"type": "yarn", "factor": 4.0, "original_max_position_embeddings": 32}))
+    assert cfg.rope_scaling.kind == "yarn" and cfg.rope_scaling.extra == {"beta_fast": 32, "beta_slow": 1, "mscale": 1.0,
+                                                                          "mscale_all_dim": 0.0}
+    m = build_model(dict(base, rope_scaling={"type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                                             "original_max_position_embeddings": 64}), "float32", "meta")
+    assert m.blocks[0].mixer.position.scaling["high_freq_factor"] == 4.0
+
+    half, theta, orig = 64, 10000.0, 8192
+    inv = 1.0 / theta ** (2.0 * torch.arange(half, dtype=torch.float64) / (2 * half))
+    new, mag = SCALINGS["llama3"](inv, {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                                        "original_max_position_embeddings": orig}, 131072)
+    wavelen = 2 * math.pi / inv
+    assert mag == 1.0
+    assert torch.equal(new[wavelen < orig / 4.0], inv[wavelen < orig / 4.0])
+    assert torch.allclose(new[wavelen > orig], inv[wavelen > orig] / 8.0, rtol=1e-12)
+    ratio = new / inv
+    assert (ratio[1:] <= ratio[:-1] + 1e-12).all() and ratio.min() >= 1 / 8.0 - 1e-12 and ratio.max() <= 1.0
+
+    new, mag = SCALINGS["yarn"](inv, {"factor": 4.0, "original_max_position_embeddings": 4096}, 16384, theta)
+    ratio = new / inv
+    assert ratio[0] == 1.0 and abs(float(ratio[-1]) - 0.25) < 1e-12 and (ratio[1:] <= ratio[:-1] + 1e-12).all()
+    assert abs(mag - (0.1 * math.log(4.0) + 1.0)) < 1e-12
+    same, one = SCALINGS["yarn"](inv, {"factor": 1.0, "original_max_position_embeddings": 4096}, 4096, theta)
+    assert torch.allclose(same, inv, rtol=1e-12) and one == 1.0
+    _, both = SCALINGS["yarn"](inv, {"factor": 4.0, "original_max_position_embeddings": 4096, "mscale": 0.7,
+                                     "mscale_all_dim": 0.7}, 16384, theta)
+    assert both == 1.0

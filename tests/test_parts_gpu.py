@@ -445,16 +445,27 @@ def test_toy_feed_forward_with_routing(tmp_path):
     assert rel_err(drv.request_logits("b", 20), plain(b)) < 1e-4
 
 
-def test_a_position_encoding_registered_from_outside(tmp_path):
+def test_a_position_encoding_and_an_output_head_registered_from_outside(tmp_path):
     """Another position encoding, defined here with a tensor of its own (a learned vector per
-    position added to every q and k head): registered, named in a layer, loaded by name and stepped in
-    portions and batches, without a change to the mixer or the step function."""
+    position added to every q and k head), and another output head (logits capped by a tanh):
+    registered, named in the model's description, loaded by name and stepped in portions and
+    batches, without a change to the mixer, the model or the step function."""
     from safetensors.torch import save_file
     from infinilm_amd import kernels
     from infinilm_amd.config import HeadSpec, LayerRun, LayerSpec, ModelSpec, PartSpec, register_architecture
     from infinilm_amd.engine.loading import build_model
-    from infinilm_amd.parts import Param, PositionEncoding, register_position_encoding
+    from infinilm_amd.parts import Param, PositionEncoding, register_head, register_position_encoding
+    from infinilm_amd.parts.ends import LinearHead
     from helpers import Driver
+
+    @register_head("toy_capped")
+    class ToyCappedHead(LinearHead):
+        def __init__(self, vocab_size, hidden_size, scale, cap, ctx):
+            super().__init__(vocab_size, hidden_size, scale, ctx)
+            self.cap = float(cap)
+
+        def forward(self, x):
+            return self.cap * torch.tanh(super().forward(x) / self.cap)
 
     @register_position_encoding("toy_learned_offsets")
     class ToyLearnedOffsets(PositionEncoding):
@@ -484,7 +495,7 @@ def test_a_position_encoding_registered_from_outside(tmp_path):
         names = {"norm1": "ln1", "mixer": "att", "norm2": "ln2", "ffn": "ffn"}
         layers = [LayerSpec(f"l.{i}", "pre_norm", {"norm1": norm, "mixer": att, "norm2": norm, "ffn": ffn}, names, 1.0) for i in range(2)]
         return ModelSpec("ToyOffsetsLM", V, H, MAXP, "emb", 1.0, layers, [LayerRun(0, 0), LayerRun(1, 1)], norm, "ln_f",
-                         HeadSpec("head", 1.0, True))
+                         HeadSpec("head", 0.5, True, kind="toy_capped", params={"cap": 3.0}))
 
     register_architecture(["ToyOffsetsLM"], dict, build_spec)
     cfg = {"architectures": ["ToyOffsetsLM"], "torch_dtype": "float32"}
@@ -516,9 +527,10 @@ def test_a_position_encoding_registered_from_outside(tmp_path):
             x = x + P.plain_linear(P.plain_attention(q, k, v, d ** -0.5).reshape(n, nh * d), Wd[p + "att.o_proj.weight"])
             h = P.plain_rmsnorm(x, Wd[p + "ln2.weight"], 1e-6)
             x = x + P.plain_mlp(h, Wd[p + "ffn.gate_proj.weight"], Wd[p + "ffn.up_proj.weight"], Wd[p + "ffn.down_proj.weight"], 1.0)
-        return P.plain_linear(P.plain_rmsnorm(x, Wd["ln_f.weight"], 1e-6), Wd["emb.weight"])
+        return 3.0 * torch.tanh(P.plain_linear(P.plain_rmsnorm(x, Wd["ln_f.weight"], 1e-6), Wd["emb.weight"], None, 0.5) / 3.0)
 
     drv = Driver(mdir, "float32", num_pages=16, page_size=8, max_requests=2)
+    assert drv.model.head_is_tied and type(drv.model.output_head).__name__ == "ToyCappedHead"
     g2 = torch.Generator().manual_seed(5)
     a, b = (torch.randint(0, V, (n,), generator=g2).tolist() for n in (61, 18))
     drv.step([("a", a[:30])])
