@@ -203,6 +203,52 @@ gemm_skinny_resident_kernel(TC* __restrict__ C, const bf16* __restrict__ X, cons
     }
 }
 
+// 1 / sqrt(mean(r^2) + eps) of a row from the partial sums of squares a producer left (gemm_tail.hip:
+// SS[tile][32]), for a product whose X is that producer's r * w, not yet divided: the division is one
+// number a row and is applied to the sums in the epilogue.  In three pieces, so that nothing waits:
+//   SK_SCALE_LOAD   before the main loop: a thread takes four rows (one 16-byte load a tile) of the tiles
+//                   c, c + C, c + 2C, ... (C = threads / (4 MG) chunks); the loads fly with the first W tile
+//   SK_SCALE_PUT    in the first round, before the barrier the reduction of the tile has anyway: the chunks of
+//                   a wave are added by shuffles, the wave's sums go to LDS `ssr[WAVES][32]`
+//   SK_SCALE_GET    after that barrier: the waves' sums in wave order
+// The order of the sum depends on the number of tiles alone.
+#define SK_SCALE_LOAD(SS_, TILES_)                                                                \
+    float4 ss_sum = make_float4(0.f, 0.f, 0.f, 0.f);                                              \
+    if ((SS_) != nullptr) {                                                                       \
+        constexpr int Q_ = 4 * MG, C_ = WAVES * 64 / Q_;                                          \
+        const float4* sp = reinterpret_cast<const float4*>(SS_) + threadIdx.x % Q_;               \
+        int tl = threadIdx.x / Q_;                                                                \
+        for (; tl + 3 * C_ < (TILES_); tl += 4 * C_) {                                            \
+            const float4 v0 = sp[(size_t)tl * 8], v1 = sp[(size_t)(tl + C_) * 8];                 \
+            const float4 v2 = sp[(size_t)(tl + 2 * C_) * 8], v3 = sp[(size_t)(tl + 3 * C_) * 8];  \
+            ss_sum.x += (v0.x + v1.x) + (v2.x + v3.x);                                            \
+            ss_sum.y += (v0.y + v1.y) + (v2.y + v3.y);                                            \
+            ss_sum.z += (v0.z + v1.z) + (v2.z + v3.z);                                            \
+            ss_sum.w += (v0.w + v1.w) + (v2.w + v3.w);                                            \
+        }                                                                                         \
+        for (; tl < (TILES_); tl += C_) {                                                         \
+            const float4 v0 = sp[(size_t)tl * 8];                                                 \
+            ss_sum.x += v0.x; ss_sum.y += v0.y; ss_sum.z += v0.z; ss_sum.w += v0.w;               \
+        }                                                                                         \
+    }
+#define SK_SCALE_PUT(SS_)                                                                         \
+    if ((SS_) != nullptr) {                                                                       \
+        constexpr int Q_ = 4 * MG;                                                                \
+        _Pragma("unroll") for (int o = Q_; o < 64; o <<= 1) {                                     \
+            ss_sum.x += __shfl_xor(ss_sum.x, o, 64);                                              \
+            ss_sum.y += __shfl_xor(ss_sum.y, o, 64);                                              \
+            ss_sum.z += __shfl_xor(ss_sum.z, o, 64);                                              \
+            ss_sum.w += __shfl_xor(ss_sum.w, o, 64);                                              \
+        }                                                                                         \
+        if ((threadIdx.x & 63) < Q_) *reinterpret_cast<float4*>(&ssr[threadIdx.x >> 6][(threadIdx.x % Q_) * 4]) = ss_sum; \
+    }
+#define SK_SCALE_GET(RSTD_, SS_, EPS_, WIDTH_, ROW_)                                              \
+    if ((SS_) != nullptr) {                                                                       \
+        float tot = 0.f;                                                                          \
+        _Pragma("unroll") for (int c = 0; c < WAVES; ++c) tot += ssr[c][ROW_];                    \
+        RSTD_ = 1.0f / sqrtf(tot / (float)(WIDTH_) + (EPS_));                                     \
+    }
+
 // The fused gate/up projection of a feed-forward with the SwiGLU in its epilogue (few rows of X):
 // W holds the gate rows [0, I) and the up rows [I, 2I).  A tile of 16 W rows is the gate rows and the
 // up rows of the same 8 outputs, so the thread that reduces gate (m, n) also reduces up (m, n) and
@@ -213,9 +259,11 @@ template <int WAVES, int KSTEPS, int MG>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_gateup_swiglu_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
                           const bf16* __restrict__ bias, int M, int I, int K, int lda, int ldw, int ldc, int ntiles,
-                          int ks) {
+                          int ks, const float* __restrict__ SS, int ss_tiles, float eps) {
+    // SS != null: X is r * w of a norm whose division is still to come (see SK_ROW_SCALE)
     static_assert(WAVES * 64 >= 128 * MG, "one reducing thread an output");
     __shared__ float part[2][MG][WAVES][64][4];
+    __shared__ __attribute__((aligned(16))) float ssr[WAVES][32];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, q = lane >> 4;
     const int s0 = wave * ks;
@@ -256,6 +304,9 @@ gemm_gateup_swiglu_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, cons
     const int et = threadIdx.x < 128 * MG ? threadIdx.x : 0;
     const int eg = et >> 7, m = eg * 16 + (et & 15), j = (et & 127) >> 4;
     const int gl = (j >> 2) * 16 + (et & 15), ge = j & 3;   // lane and element of the gate sum; up: lane + 32
+    SK_SCALE_LOAD(SS, ss_tiles)
+    float rstd = 1.0f;
+    bool first = true;
     int buf = 0;
     for (; tile < ntiles; tile += gridDim.x) {
         f32x4 acc[MG];
@@ -276,7 +327,10 @@ gemm_gateup_swiglu_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, cons
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int g = 0; g < MG; ++g) *reinterpret_cast<f32x4*>(&part[buf][g][wave][lane][0]) = acc[g];
+        if (first) SK_SCALE_PUT(SS)
         __syncthreads();
+        if (first) SK_SCALE_GET(rstd, SS, eps, K, m < 32 ? m : 0)
+        first = false;
         const int n = tile * 8 + j;
         if (threadIdx.x < 128 * MG && n < I && m < M) {
             float vg = 0.f, vu = 0.f;
@@ -285,6 +339,8 @@ gemm_gateup_swiglu_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, cons
                 vg += part[buf][eg][w][gl][ge];
                 vu += part[buf][eg][w][gl + 32][ge];
             }
+            vg *= rstd;
+            vu *= rstd;
             if (bias != nullptr) {
                 vg += to_f32(bias[n]);
                 vu += to_f32(bias[n + I]);
@@ -305,9 +361,10 @@ template <int WAVES, int KSTEPS, int MG>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_gateup_swiglu_pair_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
                           const bf16* __restrict__ bias, int M, int I, int K, int lda, int ldw, int ldc, int ntiles,
-                          int ks) {
+                          int ks, const float* __restrict__ SS, int ss_tiles, float eps) {
     static_assert(WAVES * 64 >= 256 * MG, "one reducing thread an output");
     __shared__ float part[2][MG][WAVES][64][4];
+    __shared__ __attribute__((aligned(16))) float ssr[WAVES][32];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, q = lane >> 4;
     const int s0 = wave * ks;
@@ -347,6 +404,9 @@ gemm_gateup_swiglu_pair_kernel(bf16* __restrict__ C, const bf16* __restrict__ X,
     const int et = threadIdx.x < 256 * MG ? threadIdx.x : 0;
     const int eg = et >> 8, e = et & 3, l = (et & 255) >> 2;
     const int m = eg * 16 + (l & 15);
+    SK_SCALE_LOAD(SS, ss_tiles)
+    float rstd = 1.0f;
+    bool first = true;
     int buf = 0;
     for (; tile < ntiles; tile += gridDim.x) {
         const int n = tile * 16 + (l >> 4) * 4 + e;
@@ -372,11 +432,15 @@ gemm_gateup_swiglu_pair_kernel(bf16* __restrict__ C, const bf16* __restrict__ X,
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int g = 0; g < MG; ++g) *reinterpret_cast<f32x4*>(&part[buf][g][wave][lane][0]) = acc[g];
+            if (first) SK_SCALE_PUT(SS)
             __syncthreads();
+            if (first) SK_SCALE_GET(rstd, SS, eps, K, m < 32 ? m : 0)
+            first = false;
             float v = 0.f;
             if (threadIdx.x < 256 * MG) {
 #pragma unroll
                 for (int w = 0; w < WAVES; ++w) v += part[buf][eg][w][l][e];
+                v *= rstd;
                 if (bias != nullptr && writer) v += to_f32(bias[n + hf * I]);
             }
             val[hf] = to_f32(from_f32<bf16>(v));
@@ -485,8 +549,12 @@ extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void
 }
 
 // act [M, ldc] = silu(X Wg^T + bg) * (X Wu^T + bu) with W = [Wg; Wu] of 2 I rows (bias of 2 I entries or null).
+// ss != null: X is r * w of the RMS norm before the projection, not yet divided by the rows' root mean square, and
+// ss [ss_tiles][32] holds partial sums of squares of the rows of r (what ilm_gemm_tail leaves): the kernel adds them
+// up and applies 1 / sqrt(sum / K + eps) to its sums (K is also the norm's width).
 extern "C" int ilm_gemm_gateup_swiglu(void* C, int ldc, const void* X, int lda, const void* W, int ldw, const void* bias,
-                                      int M, int I, int K, hipStream_t stream) {
+                                      int M, int I, int K, const void* ss, int ss_tiles, float eps, hipStream_t stream) {
+    ILM_REQUIRE(ss == nullptr || ss_tiles > 0, "gemm_gateup_swiglu: no tiles of partial sums");
     ILM_REQUIRE(M > 0 && M <= 32 && I > 0 && K > 0, "gemm_gateup_swiglu: needs 1 <= M <= 32, got M=%d I=%d K=%d", M, I, K);
     ILM_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldc >= I,
                 "gemm_gateup_swiglu: K=%d lda=%d ldw=%d ldc=%d", K, lda, ldw, ldc);
@@ -501,7 +569,7 @@ extern "C" int ilm_gemm_gateup_swiglu(void* C, int ldc, const void* X, int lda, 
         const int grid = ntiles < num_cus() * PER_CU ? ntiles : num_cus() * PER_CU;                         \
         KERNEL<WV, KS, MGR><<<grid, WV * 64, 0, stream>>>(                                                  \
             (bf16*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, I, K, lda, ldw, ldc, ntiles,    \
-            (ksteps + WV - 1) / WV);                                                                        \
+            (ksteps + WV - 1) / WV, (const float*)ss, ss_tiles, eps);                                       \
     }
 #define GU_CASE(WV, KS, MGR, PER_CU)                                                       \
     {                                                                                      \

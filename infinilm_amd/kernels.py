@@ -387,13 +387,69 @@ USE_GATEUP_SWIGLU = os.environ.get("INFINILM_AMD_GATEUP_SWIGLU", "1") == "1"
 USE_GATEUP_WIDE = os.environ.get("INFINILM_AMD_GATEUP_WIDE", "1") == "1"
 
 
-def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+# Rows up to which the projection that ends a branch takes the residual sum and the first half of the next
+# norm into its epilogue (gemm_tail.hip); 0: never
+TAIL_MAX_ROWS = int(os.environ.get("INFINILM_AMD_TAIL_ROWS", "16"))
+TAIL_SS_ROWS = 32   # rows of a tile's record of partial sums of squares (ilm_gemm_tail_ss_rows())
+
+
+def _mfma_operands_ok(x: torch.Tensor, w: torch.Tensor, K: int) -> bool:
+    return (x.dtype == BF16 and w.dtype == BF16 and x.is_cuda and w.shape[1] == K and K % 8 == 0 and x.stride(1) == 1
+            and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
+def tail_ok(rows: int, w: torch.Tensor, bias: Optional[torch.Tensor], norm_w: torch.Tensor, dtype: torch.dtype) -> bool:
+    """Whether `gemm_tail` takes a product of `rows` rows with the weight w [N, K] (see there)."""
+    N, K = w.shape
+    return (not FORCE_BASIC and dtype == BF16 and w.dtype == BF16 and 0 < rows <= min(TAIL_MAX_ROWS, 32)
+            and (K <= 4096 or (rows <= 16 and K <= 8192)) and K % 8 == 0 and w.stride(1) == 1 and w.stride(0) % 8 == 0
+            and w.data_ptr() % 16 == 0 and norm_w.shape == (N,) and norm_w.dtype in (BF16, F32) and norm_w.is_contiguous()
+            and (bias is None or (bias.shape == (N,) and bias.dtype == BF16 and bias.is_contiguous())))
+
+
+def gemm_tail(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], alpha: float, residual: torch.Tensor,
+              norm_w: torch.Tensor):
+    """The projection that ends a branch, with the residual sum and the first half of the norm after it
+    in its epilogue: residual += alpha * (x w^T + bias) in place (float32 [M, N]); returns (xw, ss) with
+    xw = bfloat16(residual * norm_w) [M, N], not yet divided by the rows' root mean square, and ss
+    [ceil(N / 16), 32] partial sums of squares of the residual's rows, which the consumer of xw adds up
+    (`gateup_swiglu_gemm(..., row_ss=ss, eps=...)`).  For what `tail_ok` accepts."""
+    M, K = x.shape
+    N = w.shape[0]
+    _dev(x, w, bias, residual, norm_w)
+    if not (tail_ok(M, w, bias, norm_w, x.dtype) and _mfma_operands_ok(x, w, K)):
+        raise KernelError(f"gemm_tail does not take {tuple(x.shape)} x {tuple(w.shape)}^T")
+    if residual.dtype != F32 or tuple(residual.shape) != (M, N) or residual.stride(1) != 1:
+        raise KernelError("the residual stream is a float32 tensor with dense rows of the product's width")
+    xw = torch.empty((M, N), dtype=BF16, device=x.device)
+    ss = torch.empty((-(-N // 16), TAIL_SS_ROWS), dtype=F32, device=x.device)
+    _run("ilm_gemm_tail", residual.data_ptr(), residual.stride(0), xw.data_ptr(), xw.stride(0), ss.data_ptr(), x.data_ptr(),
+         x.stride(0), w.data_ptr(), w.stride(0), _ptr(bias), norm_w.data_ptr(), _dt(norm_w), float(alpha), M, N, K, _stream())
+    return xw, ss
+
+
+def gateup_resident_ok(rows: int, w: torch.Tensor) -> bool:
+    """Whether the gate/up kernel that keeps X in registers takes `rows` rows with the weight w [2I, K]."""
+    K = w.shape[1]
+    return (USE_GATEUP_SWIGLU and not FORCE_BASIC and w.dtype == BF16 and _few_rows(rows, K) and K <= 8192 and K % 8 == 0
+            and w.shape[0] % 2 == 0 and w.stride(1) == 1 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
+                       row_ss: Optional[torch.Tensor] = None, eps: float = 0.0) -> Optional[torch.Tensor]:
     """silu(x Wg^T + bg) * (x Wu^T + bu) for few rows in bfloat16, W = [Wg; Wu]: the fused gate/up
     projection with the SwiGLU in its epilogue, [M, I] (up to 32 rows with X in registers, up to 64 with X
     through LDS).  None where no kernel applies (more rows, float32): the caller then runs the projection
-    and the activation."""
+    and the activation.  `row_ss`: x is what `gemm_tail` left (residual * norm weight) and row_ss its
+    partial sums of squares: the rows' division by sqrt(mean square + eps) happens in this kernel's
+    epilogue (only the kernel with X in registers does that: `gateup_resident_ok`)."""
     M, K = x.shape
     resident = _few_rows(M, K) and K <= 8192
+    if row_ss is not None:
+        if not (resident and gateup_resident_ok(M, w) and _mfma_operands_ok(x, w, K) and row_ss.dtype == F32
+                and row_ss.dim() == 2 and row_ss.shape[1] == TAIL_SS_ROWS and row_ss.is_contiguous() and row_ss.is_cuda):
+            raise KernelError("a product with the norm's division in its epilogue needs the few-rows gate/up kernel")
     # 17 to 64 rows that do not fit the registers: X through LDS, W streamed over the whole K by every wave
     # (64 rows at the 8B shape: 52 us against 62 + 5 for the vendor library's product and the activation kernel)
     wide = USE_GATEUP_WIDE and not resident and 16 < M <= 64
@@ -407,8 +463,12 @@ def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
     if bias is not None and (bias.shape != (2 * I,) or bias.dtype != BF16 or not bias.is_contiguous()):
         raise KernelError("bias does not fit the fused gate/up projection")
     out = torch.empty((M, I), dtype=BF16, device=x.device)
-    _run("ilm_gemm_gateup_swiglu" if resident else "ilm_gemm_gateup_wide", out.data_ptr(), out.stride(0), x.data_ptr(),
-         x.stride(0), w.data_ptr(), w.stride(0), _ptr(bias), M, I, K, _stream())
+    if resident:
+        _run("ilm_gemm_gateup_swiglu", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
+             _ptr(bias), M, I, K, _ptr(row_ss), 0 if row_ss is None else row_ss.shape[0], float(eps), _stream())
+    else:
+        _run("ilm_gemm_gateup_wide", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
+             _ptr(bias), M, I, K, _stream())
     return out
 
 

@@ -46,7 +46,9 @@ class GQAttention(Mixer):
     def cache_need(self):
         return PagedKV(self.nkv, self.d, self.window)
 
-    def forward(self, x: torch.Tensor, batch, cache_view) -> torch.Tensor:
+    takes_tail = True
+
+    def forward(self, x: torch.Tensor, batch, cache_view, tail=None):
         pe = self.position
         pe.check(batch)
         qkv = None
@@ -60,4 +62,8 @@ class GQAttention(Mixer):
         o = kernels.paged_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,
                                     batch.positions, self.nh, self.nkv, self.d, self.scale, self.window,
                                     batch.max_total_len, batch.att_tiles, batch.att_single_rows)
+        if tail is not None:   # the output projection adds into the residual stream itself, where its kernel can
+            deferred = self.o_proj.forward_tail(o, tail)
+            if deferred is not None:
+                return deferred
         return self.o_proj.forward(o, allow_parts=True)

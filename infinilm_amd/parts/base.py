@@ -70,12 +70,40 @@ class ResidualStream:
         self.pending_scale = scale
 
 
+@dataclass
+class NormTail:
+    """An offer to the part before a norm (an arrangement makes it when the norm, the part before and
+    the part after all can): add your branch into `residual` yourself (times `scale`) and return a
+    `DeferredNorm` instead of the branch; the norm's kernel is then not run."""
+    residual: torch.Tensor      # float32 [T, hidden], updated in place
+    scale: float
+    weight: torch.Tensor        # the norm's weight
+    eps: float
+
+
+@dataclass
+class DeferredNorm:
+    """A norm's output up to one number a row: `x` = residual * weight in the activations' dtype, and
+    partial sums of squares of the residual's rows (`sumsq` [tiles, 32]), from which the consumer
+    forms 1 / sqrt(mean square + eps) and applies it to its own sums."""
+    x: torch.Tensor
+    sumsq: torch.Tensor
+    eps: float
+
+
 class Norm(Part):
     def forward(self, stream: ResidualStream) -> torch.Tensor:
         raise NotImplementedError
 
+    def tail(self, stream: ResidualStream, scale: float, rows: int) -> Optional[NormTail]:
+        """The offer for the part before this norm, or None (see NormTail)."""
+        return None
+
 
 class Mixer(Part):
+    """`takes_tail`: forward accepts `tail=NormTail` and may answer with a DeferredNorm."""
+    takes_tail = False
+
     def cache_need(self):
         return None
 
@@ -84,6 +112,10 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    def takes_deferred(self, rows: int) -> bool:
+        """Whether forward accepts a DeferredNorm of `rows` rows as x."""
+        return False
+
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
         raise NotImplementedError
 

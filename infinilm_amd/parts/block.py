@@ -9,7 +9,7 @@ from __future__ import annotations
 from typing import Dict
 
 from ..config.spec import LayerSpec
-from .base import BuildContext, Param, ResidualStream
+from .base import BuildContext, DeferredNorm, Param, ResidualStream
 from .registry import ARRANGEMENTS, build_feed_forward, build_mixer, build_norm, register_arrangement
 
 
@@ -38,8 +38,20 @@ class PreNormBlock:
 
     def forward(self, stream: ResidualStream, batch, cache_view) -> None:
         x = self.norm1.forward(stream)
-        stream.push(self.mixer.forward(x, batch, cache_view), self.residual_scale)
-        x = self.norm2.forward(stream)
+        # Few rows (decoded tokens): where the mixer's last projection, the second norm and the feed-forward
+        # all can, the projection adds into the residual stream itself and the norm's kernel is not run
+        # (see NormTail).  Not while intermediate values are dumped: they are taken between the kernels.
+        tail = None
+        if self.mixer.takes_tail and batch.taps is None:
+            tail = self.norm2.tail(stream, self.residual_scale, x.shape[0])
+            if tail is not None and not self.ffn.takes_deferred(x.shape[0]):
+                tail = None
+        y = self.mixer.forward(x, batch, cache_view) if tail is None else self.mixer.forward(x, batch, cache_view, tail=tail)
+        if isinstance(y, DeferredNorm):
+            x = y
+        else:
+            stream.push(y, self.residual_scale)
+            x = self.norm2.forward(stream)
         stream.push(self.ffn.forward(x, batch), self.residual_scale)
 
 

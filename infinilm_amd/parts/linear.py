@@ -12,7 +12,7 @@ from typing import Dict, Optional, Sequence
 import torch
 
 from .. import kernels
-from .base import BuildContext, Param
+from .base import BuildContext, DeferredNorm, NormTail, Param
 
 
 class FusedLinear:
@@ -42,6 +42,15 @@ class FusedLinear:
         """`allow_parts`: the result may come as float32 parts [P, T, out] still to be summed; only for a
         result that goes straight into `ResidualStream.push` (the next norm's kernel sums them)."""
         return kernels.gemm(x, self.weight, self.bias, alpha, out_dtype, allow_parts=allow_parts)
+
+
+    def forward_tail(self, x: torch.Tensor, tail: NormTail) -> Optional[DeferredNorm]:
+        """The projection with the residual sum and the first half of the following norm in its epilogue
+        (`kernels.gemm_tail`), or None where that kernel does not take the shapes."""
+        if not kernels.tail_ok(x.shape[0], self.weight, self.bias, tail.weight, x.dtype):
+            return None
+        xw, ss = kernels.gemm_tail(x, self.weight, self.bias, tail.scale, tail.residual, tail.weight)
+        return DeferredNorm(xw, ss, tail.eps)
 
 
 class Linear(FusedLinear):

@@ -10,7 +10,7 @@ from typing import Dict
 import torch
 
 from .. import kernels
-from .base import BuildContext, FeedForward, Param
+from .base import BuildContext, DeferredNorm, FeedForward, Param
 from .linear import FusedLinear, Linear
 from .registry import register_feed_forward
 
@@ -27,7 +27,13 @@ class SwiGLU(FeedForward):
         out.update(self.down.named_parameters())
         return out
 
-    def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
+    def takes_deferred(self, rows: int) -> bool:
+        return kernels.gateup_resident_ok(rows, self.gate_up.weight)
+
+    def forward(self, x, batch) -> torch.Tensor:
+        if isinstance(x, DeferredNorm):   # the norm's division happens in the gate/up kernel's epilogue
+            act = kernels.gateup_swiglu_gemm(x.x, self.gate_up.weight, self.gate_up.bias, row_ss=x.sumsq, eps=x.eps)
+            return self.down.forward(act, allow_parts=True)
         act = kernels.gateup_swiglu_gemm(x, self.gate_up.weight, self.gate_up.bias)   # few rows: activation in the epilogue
         if act is not None:
             return self.down.forward(act, allow_parts=True)

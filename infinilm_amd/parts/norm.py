@@ -12,7 +12,7 @@ from typing import Dict
 import torch
 
 from .. import kernels
-from .base import BuildContext, Norm, Param, ResidualStream
+from .base import BuildContext, Norm, NormTail, Param, ResidualStream
 from .registry import register_norm
 
 
@@ -29,6 +29,11 @@ class RMSNorm(Norm):
 
     def named_parameters(self) -> Dict[str, Param]:
         return {"weight": Param(self.weight, keep_f32=True, replace=self._set_weight, neutral=1.0)}
+
+    def tail(self, stream: ResidualStream, scale: float, rows: int):
+        if stream.pending is not None or self.dtype != torch.bfloat16 or rows > kernels.TAIL_MAX_ROWS:
+            return None
+        return NormTail(stream.residual, float(scale), self.weight, self.eps)
 
     def forward(self, stream: ResidualStream) -> torch.Tensor:
         x = kernels.add_rmsnorm(stream.residual, stream.pending, self.weight, stream.pending_scale, self.eps,

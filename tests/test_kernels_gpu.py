@@ -294,6 +294,49 @@ def test_gate_up_projection_with_the_activation_in_its_epilogue(K, M, I, Kd, bia
         assert K.gateup_swiglu_gemm(dev(big), dev(w), dev(b)) is None                  # too many rows
 
 
+@pytest.mark.parametrize("M,Ko,H,I,bias,wdt", [(8, 4096, 4096, 16384, False, torch.bfloat16), (3, 96, 80, 200, True, torch.float32),
+                                               (16, 1032, 328, 331, True, torch.bfloat16), (1, 2304, 2304, 5760, False, torch.float32),
+                                               (20, 200, 96, 50, False, torch.float32), (32, 4096, 1024, 4096, True, torch.bfloat16),
+                                               (5, 8192, 72, 61, False, torch.bfloat16)])
+def test_branch_tail_and_deferred_norm(K, monkeypatch, M, Ko, H, I, bias, wdt):
+    """The output projection with the residual sum and the first half of the next norm in its epilogue,
+    and the gate/up projection that finishes that norm in its own: together they equal
+    residual += alpha * (x Wo^T + b); swiglu(rmsnorm(residual) Wgu^T + b) of the plain formulas."""
+    monkeypatch.setattr(K, "TAIL_MAX_ROWS", 32)
+    x, wo = _rand((M, Ko), 51, torch.bfloat16), _rand((H, Ko), 52, torch.bfloat16, scale=2.0 * Ko ** -0.5)
+    bo = _rand((H,), 53, torch.bfloat16) if bias else None
+    r = _rand((M, H), 54, scale=2.0)
+    nw = (_rand((H,), 55) * 0.2 + 1.0).to(wdt)
+    wgu = _rand((2 * I, H), 56, torch.bfloat16, scale=2.0 * H ** -0.5)
+    bgu = _rand((2 * I,), 57, torch.bfloat16) if bias else None
+    dev = lambda t: None if t is None else t.to(DEV)
+    alpha, eps = 0.37, 1e-5
+    assert K.tail_ok(M, dev(wo), dev(bo), dev(nw), torch.bfloat16) and K.gateup_resident_ok(M, dev(wgu))
+    rd = dev(r).clone()
+    xw, ss = K.gemm_tail(dev(x), dev(wo), dev(bo), alpha, rd, dev(nw))
+    act = K.gateup_swiglu_gemm(xw, dev(wgu), dev(bgu), row_ss=ss, eps=eps)
+    r_want = r.to(F64) + P.plain_linear(x.to(F64), wo.to(F64), None if bo is None else bo.to(F64), alpha)
+    _close(rd, r_want, 2e-5)
+    assert rel_sum_sq(ss, rd, M) < 1e-5
+    y = P.plain_linear(P.plain_rmsnorm(r_want, nw.to(F64), eps), wgu.to(F64), None if bgu is None else bgu.to(F64))
+    _close(act, P.plain_swiglu(y[:, :I], y[:, I:]), 1.5e-2)
+    # and against the three kernels it stands for (same places of rounding but one: r * w is rounded before the division)
+    r2 = dev(r).clone()
+    x2 = K.add_rmsnorm(r2, K.gemm(dev(x), dev(wo), dev(bo), 1.0, allow_parts=True), dev(nw), alpha, eps, torch.bfloat16)
+    two = K.gateup_swiglu_gemm(x2, dev(wgu), dev(bgu))
+    assert (act.float() - two.float()).abs().max() <= 2 ** -5 * max(float(two.float().abs().max()), 1e-6)
+    _close(rd, r2, 1e-6)
+    assert not K.tail_ok(33, dev(wo), dev(bo), dev(nw), torch.bfloat16)
+    assert not K.tail_ok(M, dev(wo), dev(bo), dev(nw), torch.float32)
+
+
+def rel_sum_sq(ss, r, M):
+    """Relative error of the rows' sums of squares formed from the tiles' partial sums."""
+    got = ss.to(F64).sum(0)[:M].cpu()
+    want = (r.to(F64) ** 2).sum(1).cpu()
+    return float(((got - want).abs() / want).max())
+
+
 def _paged(k, v, page, n_pages, seed, dtype):
     """Scatters contiguous per-request keys/values [n, nkv, d] into a paged cache with a shuffled
     block table; unused slots hold large finite garbage so that a read beyond a length shows."""
