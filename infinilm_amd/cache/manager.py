@@ -107,12 +107,16 @@ class CacheManager:
                 # keys [pages, nkv, page, d]; values transposed [pages, nkv, d, page], so that the
                 # attention kernels read consecutive keys of one dim with one load.  Zero-filled once:
                 # what a reused page holds is stale but finite, and lengths bound every read.
-                self.k[e] = torch.zeros((n, need.num_kv_heads, self.page_size, need.head_dim), dtype=dtype,
+                # One page more than the pool gives out, the last: a place for rows that belong to no request
+                # (a recorded decode step of 8 rows that serves 5 requests fills up with such rows); what
+                # lands there is never read by a request.
+                self.k[e] = torch.zeros((n + 1, need.num_kv_heads, self.page_size, need.head_dim), dtype=dtype,
                                         device=self.device)
-                self.v[e] = torch.zeros((n, need.num_kv_heads, need.head_dim, self.page_size), dtype=dtype,
+                self.v[e] = torch.zeros((n + 1, need.num_kv_heads, need.head_dim, self.page_size), dtype=dtype,
                                         device=self.device)
             elif isinstance(need, FixedState):
-                self.state[e] = torch.zeros((self.max_requests + 1,) + tuple(need.shape),
+                # row 0: the zero state; rows 1..max_requests: the slots; the last row: for rows of no request
+                self.state[e] = torch.zeros((self.max_requests + 2,) + tuple(need.shape),
                                             dtype=need.dtype or torch.float32, device=self.device)
             elif need is not None:
                 raise CacheError(f"cache entry {e}: unknown need {need!r}")
@@ -139,6 +143,14 @@ class CacheManager:
 
     def total_pages(self, group: int = 0) -> int:
         return self.groups[group].pool.num_pages if self.groups else 0
+
+    def null_page(self, group: int) -> int:
+        """The page of group `group` that belongs to no request (see the data plane above)."""
+        return self.groups[group].pool.num_pages
+
+    @property
+    def null_state_row(self) -> int:
+        return self.max_requests + 1
 
     def stats(self) -> dict:
         return {"requests": len(self.requests),

@@ -100,13 +100,17 @@ class StepRunner:
             self._copy_done[turn].record()
 
     def build_batch(self, entries: Sequence[StepEntry], min_blocks: int = 0,
-                    device_buffer: Optional[torch.Tensor] = None, defer_copy: bool = False) -> StepBatch:
+                    device_buffer: Optional[torch.Tensor] = None, defer_copy: bool = False,
+                    pad_rows: int = 0) -> StepBatch:
         """Reserves pages for every entry and lays the step's metadata out.
 
         `min_blocks` pads the block tables to a fixed width and `device_buffer` receives the
         metadata instead of a fresh tensor: a captured graph reads the same addresses at every
         replay.  `defer_copy`: the metadata stays in its staging buffer (`batch.pending_copy`): the
-        caller fills in the token ids and sends it later."""
+        caller fills in the token ids and sends it later.  `pad_rows` (steps of single tokens only):
+        that many rows of no request follow the entries' rows, so that one recorded step serves every
+        number of requests up to its size: each is a token 0 at position 0 of a sequence of its own
+        whose only page is the cache's page for such rows; its logits are computed and not returned."""
         cache = self.cache
         V = self.model.spec.vocab_size
         if not entries:
@@ -142,22 +146,27 @@ class StepRunner:
             # used by the same tokens later); nothing is half-written
             raise
 
-        R = len(entries)
-        lens = np.array([len(e.tokens) for e in entries], dtype=np.int64)
+        R_real = len(entries)
+        if pad_rows and any(len(e.tokens) != 1 for e in entries):
+            raise ValueError("rows of no request fill up steps of single tokens only")
+        R = R_real + int(pad_rows)
+        lens = np.ones(R, dtype=np.int64)
+        lens[:R_real] = [len(e.tokens) for e in entries]
         T = int(lens.sum())
-        start = np.array([cache.length(e.req_id) for e in entries], dtype=np.int64)
+        start = np.zeros(R, dtype=np.int64)
+        start[:R_real] = [cache.length(e.req_id) for e in entries]
         offsets = np.zeros(R + 1, dtype=np.int64)
         np.cumsum(lens, out=offsets[1:])
         G = len(cache.groups)
         ps = cache.page_size
         max_blocks = [max(1, min_blocks, max(len(cache.table(e.req_id, g)) for e in entries)) for g in range(G)]
-        n_want = sum(len(e.want) for e in entries)
+        n_want = sum(len(e.want) for e in entries) + int(pad_rows)
 
         # attention work lists: runs of up to TILE consecutive tokens of a request, and single tokens
         TILE = kernels.ATT_TILE_TOKENS
         tiles: List[int] = []
         singles: List[int] = []
-        for i in range(R):
+        for i in range(R_real):
             a, n = int(offsets[i]), int(lens[i])
             if n == 1:
                 singles.append(a)
@@ -186,7 +195,8 @@ class StepRunner:
             o, n = off[name]
             return h[o:o + n]
 
-        seg("token_ids")[:] = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=T)
+        seg("token_ids")[:T - pad_rows] = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=T - pad_rows)
+        seg("token_ids")[T - pad_rows:] = 0
         pos = seg("positions")
         sot = seg("seg_of_token")
         all_single = T == R
@@ -207,17 +217,23 @@ class StepRunner:
             for x in e.want:
                 w[k] = offsets[i] + x
                 k += 1
+        for i in range(R_real, R):
+            w[k] = offsets[i]
+            k += 1
         seg("att_tiles")[:] = tiles
         seg("att_singles")[:] = singles
         sin, sout = seg("state_in"), seg("state_out")
         for i, e in enumerate(entries):
             sin[i], sout[i] = cache.state_rows(e.req_id)
+        sin[R_real:] = 0
+        sout[R_real:] = cache.null_state_row
         for g in range(G):
             sl = seg(f"slots{g}")
             bt = seg(f"bt{g}").reshape(R, max_blocks[g])
             bt[:] = -1
             if all_single:
                 slot_list = []
+                bt[R_real:, 0] = cache.null_page(g)
                 for i, e in enumerate(entries):
                     table = cache.table(e.req_id, g)
                     bt[i, :len(table)] = table
@@ -226,6 +242,7 @@ class StepRunner:
                     if page < 0:
                         raise RuntimeError(f"request {e.req_id!r}: a new token falls on a page already given back")
                     slot_list.append(page * ps + p % ps)
+                slot_list += [cache.null_page(g) * ps + i % ps for i in range(pad_rows)]
                 sl[:] = slot_list
                 continue
             for i, e in enumerate(entries):
@@ -261,6 +278,7 @@ class StepRunner:
         b.block_tables = [dseg(f"bt{g}").view(R, max_blocks[g]) for g in range(G)]
         b.slots = [dseg(f"slots{g}") for g in range(G)]
         b.num_wanted = n_want
+        b.rows_of_requests = T - int(pad_rows)   # the rows after them belong to no request
         b.wants_all_rows = n_want == T and all(list(e.want) == list(range(len(e.tokens))) for e in entries)
         b.max_q_len = int(lens.max())
         b.max_total_len = int((start + lens).max())
@@ -301,11 +319,13 @@ class StepRunner:
     def _graph_key(self, entries: Sequence[StepEntry]):
         cache = self.cache
         need = max(-(-(cache.length(e.req_id) + 1) // cache.page_size) for e in entries)
-        return (len(entries), kernels.bound_pages(need))
+        return (kernels.bound_rows(len(entries)), kernels.bound_pages(need))
 
     def _graph_step(self, entries: Sequence[StepEntry], key) -> torch.Tensor:
-        """One graph per (number of requests, block-table width).  The width is rounded up
-        (`kernels.bound_pages`: 4, 6, 8, 12, 16, ... pages), so a graph serves every context up to width * page tokens; the kernels' grids are
+        """One graph per (number of rows, block-table width).  Both are rounded up: the rows to
+        `kernels.bound_rows` (1, 2, 4, 8, 16, 24, 32, 48, 64, ...: a step of 5 requests runs as one of 8, filled
+        up with rows of no request, so that requests that come and go one by one do not make a recording
+        each), the width to `kernels.bound_pages` (4, 6, 8, 12, 16, ... pages), so a graph serves every context up to width * page tokens; the kernels' grids are
         sized for that bound and bound their reads by each request's own length.  Between replays
         only the metadata buffer changes (token ids, positions, slots, block tables).  A size is
         recorded the `graph_after`-th time it comes (a recording costs about three steps, which a
@@ -313,11 +333,12 @@ class StepRunner:
         Reference: csrc/engine/compiler/paged_compiler.cpp:59-260 (one graph per decode batch size,
         inputs copied into captured buffers)."""
         cache = self.cache
-        R, width = key
+        rows, width = key
+        R = len(entries)
         slot = self._graphs.get(key)
         if slot is None:
-            buf = torch.zeros((self._graph_buffer_size(R, width),), dtype=torch.int32, device=self.device)
-            batch = self.build_batch(entries, min_blocks=width, device_buffer=buf)
+            buf = torch.zeros((self._graph_buffer_size(rows, width),), dtype=torch.int32, device=self.device)
+            batch = self.build_batch(entries, min_blocks=width, device_buffer=buf, pad_rows=rows - R)
             batch.max_total_len = width * cache.page_size     # grids are sized for the bound, not for this step
             # warm-up outside the capture (libraries set themselves up at their first call).  It runs the
             # step that the first replay runs again: keys and values are written twice with the same
@@ -347,7 +368,7 @@ class StepRunner:
                 host.numpy()[tok_off:tok_off + R] = toks
                 self._copy_to_device(dev, host, turn)
             else:
-                fresh = self.build_batch(entries, min_blocks=width, device_buffer=buf)
+                fresh = self.build_batch(entries, min_blocks=width, device_buffer=buf, pad_rows=rows - R)
                 if fresh.T != batch.T or [t.shape for t in fresh.block_tables] != [t.shape for t in batch.block_tables]:
                     raise RuntimeError("a decode step does not fit the graph captured for its size")
         graph.replay()
@@ -356,7 +377,7 @@ class StepRunner:
         self.steps += 1
         self.tokens += R
         self._prepare_next_decode(entries)
-        return logits
+        return logits[:R]
 
     def _prepare_next_decode(self, entries: Sequence[StepEntry]) -> None:
         """While the device runs the step just launched: the metadata of the same requests' next decoded
@@ -374,7 +395,7 @@ class StepRunner:
             if max(lengths) + 1 > self.model.spec.max_positions:
                 return
             b = self.build_batch([StepEntry(i, [0], [0]) for i in ids], min_blocks=key[1], device_buffer=slot[3],
-                                 defer_copy=True)
+                                 defer_copy=True, pad_rows=key[0] - len(ids))
             self._prepared = ((key, ids, cache.version), lengths, b.pending_copy)
         except (CacheError, ValueError):
             self._prepared = None   # out of pages for the guess: the real step will say so if it comes
@@ -399,7 +420,7 @@ class StepRunner:
             raise RuntimeError("no prepared decode step for these requests")
         prep, self._prepared = self._prepared, None
         key = prep[0][0]
-        R = key[0]
+        R = len(prep[0][1])
         graph, batch, logits, buf = self._graphs[key]
         dev, host, turn, tok_off = prep[2]
         if tokens_dev.dtype != torch.int32 or tokens_dev.numel() != R or tokens_dev.device != dev.device:
@@ -410,7 +431,7 @@ class StepRunner:
         graph.replay()
         self.steps += 1
         self.tokens += R
-        return logits
+        return logits[:R]
 
     def commit_ahead(self, id_tokens: Sequence) -> None:
         """The books of a step launched by `step_ahead`, now that its input tokens are known:

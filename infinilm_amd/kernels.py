@@ -506,6 +506,16 @@ def bound_pages(need: int) -> int:
     return width
 
 
+def bound_rows(rows: int) -> int:
+    """The number of rows a decode step of `rows` requests is served with when it is recorded: 1, 2, 4, 8,
+    16, 24, 32, 48, 64, 96, 128, ... (the rest are rows of no request).  The steps of these sizes stay within
+    the kernels' own row ranges (16, 32, 64 rows), so a filled-up step costs what the step itself would."""
+    b = 1
+    while b < rows:
+        b = b * 2 if b < 16 else (b * 3 // 2 if b & (b - 1) == 0 else b * 4 // 3)
+    return b
+
+
 def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple:
     """(keys a chunk, chunks) of the chunked single-token attention for `pairs` = tokens x head groups.
 
@@ -576,7 +586,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 return out
             _i32(single_rows, "single_rows")
             rows, n_single = single_rows, single_rows.numel()
-        span, nsplit = attention_chunks(int(max_total_len), page, n_single * nkv * (-(-(nh // nkv) // 16)), q.device)
+        # (the tokens counted as the recorded steps round them, so that an eager step and a replayed one cut alike)
+        span, nsplit = attention_chunks(int(max_total_len), page, bound_rows(n_single) * nkv * (-(-(nh // nkv) // 16)), q.device)
         ws_acc = ws_ml = None
         if nsplit > 1:
             # partial results of the rows served here (not of every token of the step)

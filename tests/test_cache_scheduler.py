@@ -70,7 +70,7 @@ def test_slots_pages_and_block_tables():
 def test_window_group_has_pages_of_its_own_and_gives_them_back():
     c = _cache(num_pages=6, page_size=4, needs=[PagedKV(1, 4), PagedKV(1, 4, window=6), PagedKV(2, 8)])
     assert len(c.groups) == 2 and c.group_of_entry == {0: 0, 1: 1, 2: 0}
-    assert c.k[2].shape == (6, 2, 4, 8)
+    assert c.k[2].shape == (6 + 1, 2, 4, 8) and c.null_page(0) == 6   # one page more: for rows of no request
     c.admit("a")
     for n in (5, 1, 1, 4, 1):
         c.reserve("a", n)
@@ -88,7 +88,7 @@ def test_window_group_has_pages_of_its_own_and_gives_them_back():
 
 def test_state_slots():
     c = _cache(needs=[PagedKV(1, 4), FixedState((3, 2))], max_requests=2)
-    assert c.state[1].shape == (3, 3, 2) and not c.state[1].any()
+    assert c.state[1].shape == (2 + 2, 3, 2) and not c.state[1].any() and c.null_state_row == 3   # zero row, 2 slots, row of no request
     c.admit("a")
     c.admit("b")
     ra, rb = c.state_rows("a"), c.state_rows("b")

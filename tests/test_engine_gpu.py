@@ -283,6 +283,48 @@ def test_graph_steps_with_a_changing_set_of_requests(models):
         assert r.cache.free_pages() == 48
 
 
+def test_recorded_steps_filled_up_with_rows_of_no_request(models):
+    """A recorded decode step has 1, 2, 4, 8, 16, 24, ... rows; fewer requests are served by it with the rest
+    of the rows belonging to no request.  Requests leave one by one: every step must equal the eager
+    step bit for bit, few recordings are made, and the cache's books and pages stay right."""
+    from infinilm_amd.engine.loading import load_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+
+    cfg, d, W = models[("C", "bfloat16")]
+    model = load_model(d, "bfloat16", "cuda:0")
+    n = 11
+    eager = make_runner(model, num_pages=48, page_size=16, max_requests=n)
+    graph = make_runner(model, num_pages=48, page_size=16, max_requests=n, enable_graph=True)
+    graph.graph_after = 1
+    prompts = {f"r{i}": random_tokens(cfg, 4 + 3 * i, 80 + i) for i in range(n)}
+    for r in (eager, graph):
+        for rid, p in prompts.items():
+            r.cache.admit(rid)
+        r.step([StepEntry(rid, p, []) for rid, p in prompts.items()])
+    live = list(prompts)
+    nxt = {rid: 3 + i for i, rid in enumerate(live)}
+    sizes = set()
+    for step in range(2 * n):
+        entries = [StepEntry(rid, [nxt[rid]], [0]) for rid in live]
+        le = eager.step(entries).clone()
+        torch.cuda.synchronize()
+        lg = graph.step(entries)
+        assert lg.shape == le.shape and torch.equal(le.cpu(), lg.cpu()), f"{len(live)} requests: replay differs from the eager step"
+        sizes.add(len(live))
+        nxt = {rid: int(torch.argmax(le[i])) for i, rid in enumerate(live)}
+        if step % 2 == 1 and len(live) > 1:    # a request leaves every other step
+            gone = live.pop(step % len(live))
+            for r in (eager, graph):
+                r.cache.release(gone)
+                r.cache.check()
+    assert sizes == set(range(1, n + 1))
+    assert {k[0] for k in graph._graphs} == {1, 2, 4, 8, 16}   # five recordings served eleven sizes
+    for r in (eager, graph):
+        for rid in live:
+            r.cache.release(rid)
+        assert r.cache.free_pages() == 48
+
+
 def test_graph_with_many_requests_replays_like_eager(models):
     """More than 16 decoded tokens a step: the projections go to the vendor library inside the
     captured graph; replays must still equal eager steps, several times over."""
