@@ -175,7 +175,7 @@ extern "C" int ilm_gemm_qkv_rope(void* Q, int ldq, const void* X, int lda, const
     const int total_pairs = (nh + 2 * nkv) * (d / 2);
 #define QR_CASE(WV, KS, MGR)                                                                                   \
     {                                                                                                          \
-        const int cap = qr_num_cus() * ((WV == 16 || (MGR == 2 && KS == 16)) ? 1 : 2);                         \
+        const int cap = qr_num_cus() * ((WV == 16 || (MGR == 2 && KS >= 12)) ? 1 : 2);                         \
         int ppu = (total_pairs + cap - 1) / cap;                                                               \
         if (ppu > 16) ppu = 16;                                                                                \
         const int n_units = (total_pairs + ppu - 1) / ppu;                                                     \
@@ -188,11 +188,14 @@ extern "C" int ilm_gemm_qkv_rope(void* Q, int ldq, const void* X, int lda, const
     if (M > 16) {
         if (ksteps <= 8 * 4) QR_CASE(8, 4, 2)
         else if (ksteps <= 8 * 8) QR_CASE(8, 8, 2)
+        else if (ksteps <= 8 * 12) QR_CASE(8, 12, 2)
         else QR_CASE(8, 16, 2)
     }
     else if (ksteps <= 8 * 4) QR_CASE(8, 4, 1)
     else if (ksteps <= 8 * 8) QR_CASE(8, 8, 1)
+    else if (ksteps <= 8 * 12) QR_CASE(8, 12, 1)   // (a width like 2304: 9 of 12 slots a wave instead of 5 of 8 in 16 waves)
     else if (ksteps <= 16 * 8) QR_CASE(16, 8, 1)
+    else if (ksteps <= 16 * 12) QR_CASE(16, 12, 1)
     else QR_CASE(16, 16, 1)
 #undef QR_CASE
     ILM_LAUNCH_CHECK("gemm_qkv_rope");

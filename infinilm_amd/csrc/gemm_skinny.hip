@@ -501,12 +501,15 @@ extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void
     if (mg == 2) {                                              \
         if (ksteps <= 8 * 4) SR_CASE(8, 4, 2, 2, TC)            \
         else if (ksteps <= 8 * 8) SR_CASE(8, 8, 2, 2, TC)       \
+        else if (ksteps <= 8 * 12) SR_CASE(8, 12, 2, 1, TC)     \
         else SR_CASE(8, 16, 2, 1, TC)                           \
     }                                                           \
     else if (ksteps <= 8 * 4) SR_CASE(8, 4, 1, 2, TC)           \
     else if (ksteps <= 8 * 8) SR_CASE(8, 8, 1, 2, TC)           \
+    else if (fat_waves && ksteps <= 8 * 12) SR_CASE(8, 12, 1, 2, TC) \
     else if (fat_waves) SR_CASE(8, 16, 1, 2, TC)                \
     else if (ksteps <= 16 * 8) SR_CASE(16, 8, 1, 1, TC)         \
+    else if (ksteps <= 16 * 12) SR_CASE(16, 12, 1, 1, TC)       \
     else SR_CASE(16, 16, 1, 1, TC)
         if (out_dtype == ILM_DTYPE_BF16) { SR_DISPATCH(bf16) } else { SR_DISPATCH(float) }
 #undef SR_DISPATCH
@@ -579,11 +582,14 @@ extern "C" int ilm_gemm_gateup_swiglu(void* C, int ldc, const void* X, int lda, 
     if (M > 16) {
         if (ksteps <= 8 * 4) GU_CASE(8, 4, 2, 2)
         else if (ksteps <= 8 * 8) GU_CASE(8, 8, 2, 2)
+        else if (ksteps <= 8 * 12) GU_CASE(8, 12, 2, 1)
         else GU_CASE(8, 16, 2, 1)
     }
     else if (ksteps <= 8 * 4) GU_CASE(8, 4, 1, 2)
     else if (ksteps <= 8 * 8) GU_CASE(8, 8, 1, 2)
+    else if (ksteps <= 8 * 12) GU_CASE(8, 12, 1, 2)   // (a width like 2304: 9 of 12 slots a wave instead of 9 of 16)
     else if (ksteps <= 8 * 16) GU_CASE(8, 16, 1, 2)
+    else if (ksteps <= 16 * 12) GU_CASE(16, 12, 1, 1)
     else GU_CASE(16, 16, 1, 1)
 #undef GU_LAUNCH
 #undef GU_CASE

@@ -168,11 +168,14 @@ extern "C" int ilm_gemm_tail(void* R, int ldr, void* XW, int ldxw, void* SS, con
     if (M > 16) {
         if (ksteps <= 8 * 4) GT_CASE(8, 4, 2, 2)
         else if (ksteps <= 8 * 8) GT_CASE(8, 8, 2, 2)
+        else if (ksteps <= 8 * 12) GT_CASE(8, 12, 2, 1)
         else GT_CASE(8, 16, 2, 1)
     }
     else if (ksteps <= 8 * 4) GT_CASE(8, 4, 1, 2)
     else if (ksteps <= 8 * 8) GT_CASE(8, 8, 1, 2)
+    else if (ksteps <= 8 * 12) GT_CASE(8, 12, 1, 2)
     else if (ksteps <= 8 * 16) GT_CASE(8, 16, 1, 2)
+    else if (ksteps <= 16 * 12) GT_CASE(16, 12, 1, 1)
     else GT_CASE(16, 16, 1, 1)
 #undef GT_LAUNCH
 #undef GT_CASE

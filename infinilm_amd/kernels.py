@@ -295,7 +295,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     # 65 to 208 rows on their way into the residual sum: split over K, where the vendor library leaves the
     # chip idle (measured at the 8B shapes: down projection 68 -> 36 us at 96 rows, 81 -> 39 at 128, 92 -> 44
     # at 160, 114 -> 48 at 192, 63 -> 51 at 208; o projection 22 -> 17, 25 -> 19, 32 -> 23 at 192)
-    if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS:
+    # (not for small matrices, whose few tiles leave most of the chip idle whatever the split: 0.5B shape at 128
+    # rows 2.22 against 1.96 ms a step with the library)
+    if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS and N * K >= MID_MIN_WEIGHT:
         return _gemm_mid(a, w, K, False)
     # 17 to 64 rows on their way into the residual sum: K in ranges of 1024 with the X fragments of all rows
     # in registers (o projection at 64 rows 13.1 against the library's 18.9 us, down projection 33.9
@@ -366,6 +368,7 @@ F32_FEW_ROWS = int(os.environ.get("INFINILM_AMD_F32_FEW_ROWS", "64"))
 ROWS64_SPAN = 1024   # K range of one part of the 17-to-64-rows product (ilm_gemm_rows64_span())
 ROWS64_MAX_PARTS = int(os.environ.get("INFINILM_AMD_ROWS64_PARTS", "16"))   # 0: never this kernel
 MID_MAX_ROWS = int(os.environ.get("INFINILM_AMD_MID_ROWS", "208"))  # 16: above 16 rows always the library
+MID_MIN_WEIGHT = 5 << 20   # elements of W from which the medium-rows product is used
 MID_TARGET_WGS = int(os.environ.get("INFINILM_AMD_MID_WGS", "512"))
 
 
@@ -385,6 +388,8 @@ def _gemm_mid(x: torch.Tensor, w: torch.Tensor, K: int, act: bool) -> torch.Tens
 
 USE_GATEUP_SWIGLU = os.environ.get("INFINILM_AMD_GATEUP_SWIGLU", "1") == "1"
 USE_GATEUP_WIDE = os.environ.get("INFINILM_AMD_GATEUP_WIDE", "1") == "1"
+# outputs from which the kernel with X through LDS is used (-1: 48 a compute unit; 0: always, as its tests do)
+GATEUP_WIDE_MIN_OUTPUTS = int(os.environ.get("INFINILM_AMD_GATEUP_WIDE_MIN", "-1"))
 
 
 # Rows up to which the projection that ends a branch takes the residual sum and the first half of the next
@@ -452,7 +457,10 @@ def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
             raise KernelError("a product with the norm's division in its epilogue needs the few-rows gate/up kernel")
     # 17 to 64 rows that do not fit the registers: X through LDS, W streamed over the whole K by every wave
     # (64 rows at the 8B shape: 52 us against 62 + 5 for the vendor library's product and the activation kernel)
-    wide = USE_GATEUP_WIDE and not resident and 16 < M <= 64
+    # (a workgroup takes 64 outputs: with fewer outputs than three quarters of the compute units have workgroups
+    # the library is faster - 2B-family shape, 5,760 outputs, 64 rows: 6.40 against 6.07 ms a step)
+    wide_min = GATEUP_WIDE_MIN_OUTPUTS if GATEUP_WIDE_MIN_OUTPUTS >= 0 else 48 * _num_cus(x.device)
+    wide = USE_GATEUP_WIDE and not resident and 16 < M <= 64 and w.shape[0] // 2 >= wide_min
     if not (USE_GATEUP_SWIGLU and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and x.is_cuda
             and (resident or wide) and K % 8 == 0 and w.shape[0] % 2 == 0 and w.shape[1] == K
             and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
@@ -496,6 +504,14 @@ def swiglu_gemm(gate_up: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
 _NUM_CUS: dict = {}
 
 
+def _num_cus(device) -> int:
+    """Compute units of the device (looked up once)."""
+    cus = _NUM_CUS.get(device)
+    if cus is None:
+        cus = _NUM_CUS[device] = torch.cuda.get_device_properties(device).multi_processor_count
+    return cus
+
+
 def bound_pages(need: int) -> int:
     """The block-table width a context of `need` pages is served with: 4, 6, 8, 12, 16, 24, ... (at
     most a third above the need).  The step function records one graph a width, and the attention
@@ -528,9 +544,7 @@ def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple
     At most ATT_MAX_CHUNKS chunks.  The length is first rounded up the way the step function rounds
     its graphs' block tables (`bound_pages`), so that an eager step and a replayed one cut alike."""
     bound = bound_pages(-(-max_total_len // page)) * page
-    cus = _NUM_CUS.get(device)
-    if cus is None:
-        cus = _NUM_CUS[device] = torch.cuda.get_device_properties(device).multi_processor_count
+    cus = _num_cus(device)
     steps = -(-bound // ATT_STEP)
     pairs = max(pairs, 1)
     workgroups = lambda per_chunk: pairs * -(-steps // per_chunk)

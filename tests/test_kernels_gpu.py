@@ -222,9 +222,13 @@ def test_gemm_bfloat16(K, M, N, K_, out_dtype):
                                     (48, 331, 200), (35, 50, 8200), (128, 1030, 1096), (97, 64, 72), (32, 4096, 16384),
                                     (20, 331, 12296), (27, 50, 8200), (5, 96, 5760), (30, 2304, 5760), (192, 4096, 16384), (208, 331, 4096),
                                     (150, 331, 1096), (177, 96, 200)])
-def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
+def test_gemm_split_over_k_and_its_consumer(K, monkeypatch, M, N, K_):
     """Few rows and long K: the product comes as float32 parts; add_rmsnorm sums them in order."""
     a, w = _rand((M, K_), 14, torch.bfloat16), _rand((N, K_), 15, torch.bfloat16, 0.05)
+    if M > 64 and N * K_ < K.MID_MIN_WEIGHT:
+        # a small matrix is left to the library on the engine's path; the medium-rows kernel is tested all the same
+        assert K.gemm(a.to(DEV), w.to(DEV), allow_parts=True).dtype == torch.bfloat16
+        monkeypatch.setattr(K, "MID_MIN_WEIGHT", 0)
     parts = K.gemm(a.to(DEV), w.to(DEV), allow_parts=True)
     if 16 < M <= 64 and K_ % 8 == 0:   # K ranges of 1024 (up to 32 rows with K beyond 4096: ranges of 4096)
         assert parts.shape[0] == (-(-K_ // 4096) if M <= 32 and K_ > 4096 else -(-K_ // 1024))
@@ -241,7 +245,8 @@ def test_gemm_split_over_k_and_its_consumer(K, M, N, K_):
     assert whole.dim() == 2 and whole.dtype == torch.bfloat16
     short = K.gemm(a[:, :256].contiguous().to(DEV), w[:, :256].contiguous().to(DEV), allow_parts=True)
     # short K: float32, not rounded to bfloat16 (more than 16 rows: parts)
-    assert (short.dtype == torch.float32 and short.dim() == 2) if M <= 16 else short.dim() == 3
+    # (many rows of a small matrix: the library's bfloat16 result)
+    assert (short.dtype == torch.float32 and short.dim() == 2) if M <= 16 else (short.dim() == 3 or (M > 64 and N * 256 < K.MID_MIN_WEIGHT))
     _close(whole, want, 6e-3)
     r = _rand((M, N), 16, scale=2.0)
     nw = _rand((N,), 17, torch.bfloat16) + 1
@@ -276,9 +281,13 @@ def test_swiglu_inside_the_down_projection(K, M, I, N):
                                          # 33 to 64 rows, and 17 to 32 with a long K: X through LDS
                                          (64, 16384, 4096, False), (33, 331, 1032, True), (48, 200, 96, False), (49, 4100, 520, True),
                                          (40, 5760, 2304, False), (64, 61, 8, True), (20, 96, 8200, False)])
-def test_gate_up_projection_with_the_activation_in_its_epilogue(K, M, I, Kd, bias):
+def test_gate_up_projection_with_the_activation_in_its_epilogue(K, monkeypatch, M, I, Kd, bias):
     """One kernel for silu(x Wg^T) * (x Wu^T) against the plain formula and against the projection
     followed by the activation kernel (gate and up rounded to bfloat16 at the same place)."""
+    if I < 12288 and (M > 32 or (M > 16 and Kd > 4096)):
+        # few outputs are left to the library on the engine's path (they do not fill the chip); the kernel is tested all the same
+        assert K.gateup_swiglu_gemm(_rand((M, Kd), 31, torch.bfloat16).to(DEV), _rand((2 * I, Kd), 32, torch.bfloat16).to(DEV), None) is None
+        monkeypatch.setattr(K, "GATEUP_WIDE_MIN_OUTPUTS", 0)
     x, w = _rand((M, Kd), 31, torch.bfloat16), _rand((2 * I, Kd), 32, torch.bfloat16, scale=2.0 * Kd ** -0.5)
     b = _rand((2 * I,), 33, torch.bfloat16) if bias else None
     dev = lambda t: None if t is None else t.to(DEV)
