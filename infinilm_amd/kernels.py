@@ -19,7 +19,7 @@ BF16 = torch.bfloat16
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 ATT_TILE_TOKENS = 8  # tokens per tile of the prompt-portion attention kernel (ilm_attn_tile_tokens())
 ATT_STEP = 128  # keys a workgroup of the chunked attention takes in one step (ilm_attn_mfma_step())
-ATT_MAX_CHUNKS = 64  # most chunks a context is cut into (the merge kernel walks them one after the other)
+ATT_MAX_CHUNKS = 256  # most chunks a context is cut into (a wave of the merge kernel walks a quarter of them; it takes 512)
 BASIC_CHUNK = 512    # keys a chunk of the plain attention kernel (ilm_attn_basic_chunk())
 BASIC_SPLIT = os.environ.get("INFINILM_AMD_BASIC_SPLIT", "1") == "1"   # 0: always one wave a (token, head)
 BASIC_SPLIT_WAVES = 4096   # (token, head) pairs up to which the plain kernel takes one wave a chunk
@@ -541,7 +541,7 @@ def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple
     while it still has two for each.  Measured at the 8B head shape, 4096 keys, kernel + merge:
     8 tokens 17.0 us with 256 keys a chunk (128: 18.4, 512: 20.2); 16 tokens 22.4 with 512 (256:
     24.0); 32 tokens 34.3 with 512 (256: 40.0, 1024: 36.5); 64 tokens 57.5 with 1024 (512: 60.5).
-    At most ATT_MAX_CHUNKS chunks.  The length is first rounded up the way the step function rounds
+    At most ATT_MAX_CHUNKS chunks (one token over 32,768 keys: 128 chunks of 256 keys 14.9 us, 64 of 512 18.1).  The length is first rounded up the way the step function rounds
     its graphs' block tables (`bound_pages`), so that an eager step and a replayed one cut alike."""
     bound = bound_pages(-(-max_total_len // page)) * page
     cus = _num_cus(device)

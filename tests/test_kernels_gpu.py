@@ -488,6 +488,21 @@ def test_attention_bfloat16_pages_longer_than_a_key_tile(K, nh, nkv, d, page):
     _close(out, want, 1.2e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,page,lens", [(4, 2, 64, 64, [20000, 9000]), (8, 2, 128, 256, [16500]), (3, 1, 48, 16, [5000, 3300, 70])])
+def test_attention_bfloat16_few_tokens_over_many_chunks(K, nh, nkv, d, page, lens):
+    """One or two decoded tokens over tens of thousands of keys: up to 256 chunks, merged by the kernel of
+    four waves (a quarter of the chunks each) instead of the one of one wave; a far key that dominates, a
+    window that leaves most chunks out."""
+    span, nsplit = K.attention_chunks(max(lens), page, K.bound_rows(len(lens)) * nkv, torch.device(DEV))
+    assert nsplit > 24 and nsplit <= K.ATT_MAX_CHUNKS   # the merge of four waves
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=lens, qlens=[1] * len(lens), seed=41)
+    _close(out, want, 1.2e-2)
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=lens, qlens=[1] * len(lens), seed=42, spike=True)
+    _close(out, want, 1.2e-2)
+    out, want = _attention_case(K, torch.bfloat16, nh, nkv, d, page, lens=lens, qlens=[1] * len(lens), seed=43, window=max(lens) // 2 + 77)
+    _close(out, want, 1.2e-2)
+
+
 @pytest.mark.parametrize("nh,nkv,d,page,n", [(8, 8, 64, 16, 40), (32, 2, 128, 64, 150), (4, 1, 32, 16, 120)])
 def test_attention_bfloat16_many_single_tokens(K, nh, nkv, d, page, n):
     """Many decoded tokens in one launch: the chunks get long (several 128-key steps a workgroup,
