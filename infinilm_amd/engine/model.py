@@ -9,7 +9,7 @@ computes logits at every position.
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional
+from typing import Dict, List
 
 import torch
 
