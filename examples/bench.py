@@ -148,7 +148,8 @@ def main(argv=None) -> int:
               num_blocks=max(need, 1), block_size=page, enable_graph=cfg.enable_graph,
               skip_load=cfg.skip_load or cfg.random_weights, max_num_batched_tokens=cfg.max_num_batched_tokens,
               chunk_size=cfg.chunk_size, admission=cfg.admission, seed=cfg.seed,
-              enable_prefix_caching=cfg.enable_prefix_caching, look_ahead=cfg.look_ahead)
+              enable_prefix_caching=cfg.enable_prefix_caching, look_ahead=cfg.look_ahead,
+              record_graphs_at_start=cfg.record_graphs_at_start)
     sp_kwargs = dict(temperature=cfg.temperature, top_k=cfg.top_k, top_p=cfg.top_p)
     try:
         if cfg.warmup:

@@ -26,7 +26,8 @@ def main(argv=None) -> int:
                 top_p=cfg.top_p, enable_graph=cfg.enable_graph, attn_backend=cfg.attn,
                 skip_load=cfg.skip_load or cfg.random_weights, max_num_batched_tokens=cfg.max_num_batched_tokens,
                 chunk_size=cfg.chunk_size, admission=cfg.admission, seed=cfg.seed,
-                enable_prefix_caching=cfg.enable_prefix_caching, look_ahead=cfg.look_ahead)
+                enable_prefix_caching=cfg.enable_prefix_caching, look_ahead=cfg.look_ahead,
+                record_graphs_at_start=cfg.record_graphs_at_start)
     sp = SamplingParams(temperature=cfg.temperature, top_p=cfg.top_p, top_k=cfg.top_k, max_tokens=cfg.max_new_tokens,
                         ignore_eos=cfg.ignore_eos)
     t1 = time.time()

@@ -36,6 +36,8 @@ class BaseConfig:
         ap.add_argument("--chunk-size", type=int, default=None, help="longest portion of a prompt in one step")
         ap.add_argument("--admission", type=str, default="optimistic", choices=["optimistic", "reserve_full"])
         ap.add_argument("--enable-graph", action="store_true")
+        ap.add_argument("--record-graphs-at-start", action="store_true",
+                        help="with --enable-graph: record every decode step size before the first request")
         ap.add_argument("--disable-look-ahead", dest="look_ahead", action="store_false", default=None,
                         help="with --enable-graph: wait for a step's tokens before the next step is launched")
         ap.add_argument("--disable-prefix-caching", dest="enable_prefix_caching", action="store_false", default=True,

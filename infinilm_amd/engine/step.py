@@ -113,7 +113,7 @@ class StepRunner:
         whose only page is the cache's page for such rows; its logits are computed and not returned."""
         cache = self.cache
         V = self.model.spec.vocab_size
-        if not entries:
+        if not entries and not pad_rows:
             raise ValueError("a step needs at least one entry")
         if not defer_copy:
             # prepared metadata lies in one of the two staging buffers that this step and the next take
@@ -159,7 +159,7 @@ class StepRunner:
         np.cumsum(lens, out=offsets[1:])
         G = len(cache.groups)
         ps = cache.page_size
-        max_blocks = [max(1, min_blocks, max(len(cache.table(e.req_id, g)) for e in entries)) for g in range(G)]
+        max_blocks = [max(1, min_blocks, max((len(cache.table(e.req_id, g)) for e in entries), default=0)) for g in range(G)]
         n_want = sum(len(e.want) for e in entries) + int(pad_rows)
 
         # attention work lists: runs of up to TILE consecutive tokens of a request, and single tokens
@@ -337,22 +337,7 @@ class StepRunner:
         R = len(entries)
         slot = self._graphs.get(key)
         if slot is None:
-            buf = torch.zeros((self._graph_buffer_size(rows, width),), dtype=torch.int32, device=self.device)
-            batch = self.build_batch(entries, min_blocks=width, device_buffer=buf, pad_rows=rows - R)
-            batch.max_total_len = width * cache.page_size     # grids are sized for the bound, not for this step
-            # warm-up outside the capture (libraries set themselves up at their first call).  It runs the
-            # step that the first replay runs again: keys and values are written twice with the same
-            # values, fixed-size states are put back in between
-            saved = cache.snapshot_states([e.req_id for e in entries])
-            self.model.forward(batch, cache)
-            cache.restore_states(saved)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            if self._graph_pool is None:
-                self._graph_pool = torch.cuda.graph_pool_handle()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                logits = self.model.forward(batch, cache)
-            self._graphs[key] = (graph, batch, logits, buf)
+            graph, batch, logits, buf = self._record(key, entries)
         else:
             graph, batch, logits, buf = slot
             ids = tuple(e.req_id for e in entries)
@@ -378,6 +363,58 @@ class StepRunner:
         self.tokens += R
         self._prepare_next_decode(entries)
         return logits[:R]
+
+    def _record(self, key, entries: Sequence[StepEntry]):
+        """Records the decode step of size `key` with the entries' rows first and rows of no request
+        after them (entries may be empty: a recording made before any request has come)."""
+        cache = self.cache
+        rows, width = key
+        buf = torch.zeros((self._graph_buffer_size(rows, width),), dtype=torch.int32, device=self.device)
+        batch = self.build_batch(entries, min_blocks=width, device_buffer=buf, pad_rows=rows - len(entries))
+        batch.max_total_len = width * cache.page_size     # grids are sized for the bound, not for this step
+        # warm-up outside the capture (libraries set themselves up at their first call).  It runs the
+        # step that the first replay runs again: keys and values are written twice with the same
+        # values, fixed-size states are put back in between
+        saved = cache.snapshot_states([e.req_id for e in entries])
+        self.model.forward(batch, cache)
+        cache.restore_states(saved)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        if self._graph_pool is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        with torch.cuda.graph(graph, pool=self._graph_pool):
+            logits = self.model.forward(batch, cache)
+        self._graphs[key] = (graph, batch, logits, buf)
+        return self._graphs[key]
+
+    def record_decode_graphs(self, max_rows: int, max_context: int) -> int:
+        """Records, before any request has come, the decode steps of every size that up to `max_rows`
+        requests with contexts up to `max_context` tokens can need (rows of no request stand in for the
+        requests), so that no step of a running service pays for a recording: returns how many were
+        made.  The reference records its decode graphs when the engine is built, one a batch size
+        (csrc/engine/compiler/paged_compiler.cpp:28-57, :59-260)."""
+        if not self.enable_graph or max_rows < 1:
+            return 0
+        sizes, r = [], 1
+        while True:
+            sizes.append(kernels.bound_rows(r))
+            if sizes[-1] >= max_rows:
+                break
+            r = sizes[-1] + 1
+        pages = max(1, -(-int(max_context) // self.cache.page_size)) if self.cache.groups else 1
+        widths, w = [], 1
+        while True:
+            widths.append(kernels.bound_pages(w))
+            if widths[-1] >= pages:
+                break
+            w = widths[-1] + 1
+        made = 0
+        for width in widths:
+            for rows in sizes:
+                if (rows, width) not in self._graphs:
+                    self._record((rows, width), [])
+                    made += 1
+        return made
 
     def _prepare_next_decode(self, entries: Sequence[StepEntry]) -> None:
         """While the device runs the step just launched: the metadata of the same requests' next decoded

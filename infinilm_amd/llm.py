@@ -41,6 +41,9 @@ class LLM:
     admission       "optimistic" (preempt when pages run out) | "reserve_full" (the reference's check)
     look_ahead      with enable_graph: a decode step is launched before the tokens of the one before it are
                     back on the host (None: on whenever enable_graph is)
+    record_graphs_at_start   with enable_graph: every decode step size that max_batch_size requests within the
+                    model's positions and the pool's pages can need is recorded before the first request (the
+                    reference records when the engine is built); otherwise a size is recorded the second time it comes
     enable_prefix_caching   whole pages of computed tokens stay findable for later requests that begin
                     with the same tokens (the reference's default; off where a model's cache entries
                     keep a window or a state of their own)
@@ -53,7 +56,7 @@ class LLM:
                  enable_prefix_caching: bool = True, max_num_batched_tokens: Optional[int] = None,
                  chunk_size: Optional[int] = None, admission: str = "optimistic", seed: int = 0,
                  random_weights: bool = False, random_std: float = 0.02, tokenizer=None,
-                 look_ahead: Optional[bool] = None):
+                 look_ahead: Optional[bool] = None, record_graphs_at_start: bool = False):
         if cache_type != "paged":
             raise ValueError("only the paged cache exists here (cache_type='paged')")
         if attn_backend not in ("default", "paged-attn"):
@@ -80,6 +83,11 @@ class LLM:
             tokenizer = _load_tokenizer(model_path)
         self.tokenizer = tokenizer
         self.enable_graph = enable_graph
+        if enable_graph and record_graphs_at_start:
+            reach = model.spec.max_positions
+            if runner.cache.groups:   # no request holds more than the pool has
+                reach = min(reach, min(g.pool.num_pages for g in runner.cache.groups) * block_size)
+            self.graphs_recorded_at_start = runner.record_decode_graphs(max_batch_size, reach)
         self.engine = LLMEngine(runner, max_num_seqs=max_batch_size, max_num_batched_tokens=max_num_batched_tokens,
                                 chunk_size=chunk_size, policy=admission, seed=seed, tokenizer=tokenizer,
                                 look_ahead=look_ahead)

@@ -325,6 +325,30 @@ def test_recorded_steps_filled_up_with_rows_of_no_request(models):
         assert r.cache.free_pages() == 48
 
 
+def test_decode_steps_recorded_before_the_first_request(models):
+    """`record_graphs_at_start`: every decode step size that the batch limit, the model's positions and the pool
+    allow is recorded from rows of no request when the engine is built; the requests that come later find
+    their recordings (none is added), replay them with their own rows first, and generate what the plain
+    implementation generates.  Nothing of the cache is held or written outside the page for such rows."""
+    from infinilm_amd import LLM, SamplingParams
+
+    cfg, d, W = models[("A", "float32")]
+    llm = LLM(d, dtype="float32", num_blocks=16, block_size=16, max_batch_size=5, enable_graph=True,
+              record_graphs_at_start=True, enable_prefix_caching=False)
+    runner = llm.engine.runner
+    # rows 1, 2, 4, 8 (five requests run as eight rows); widths 4, 6, 8 pages (128 positions: 8 pages of 16)
+    assert set(runner._graphs) == {(r, w) for r in (1, 2, 4, 8) for w in (4, 6, 8)}
+    assert llm.graphs_recorded_at_start == 12
+    assert runner.cache.free_pages() == 16 and not runner.cache.requests
+    prompts = [random_tokens(cfg, n, 300 + n) for n in (3, 40, 17, 9, 1)]
+    outs = llm.generate(prompt_token_ids=prompts, sampling_params=SamplingParams(top_k=1, max_tokens=20, ignore_eos=True))
+    assert len(runner._graphs) == 12                      # no step had to record
+    assert runner.cache.free_pages() == 16
+    for p, o in zip(prompts, outs):
+        assert o.outputs[0].token_ids == P.plain_greedy(cfg, W, p, 20)
+    llm.close()
+
+
 def test_graph_with_many_requests_replays_like_eager(models):
     """More than 16 decoded tokens a step: the projections go to the vendor library inside the
     captured graph; replays must still equal eager steps, several times over."""
