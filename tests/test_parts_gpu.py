@@ -606,12 +606,17 @@ def test_a_model_without_paged_keys_runs_through_the_entry_point_with_graphs(tmp
     g2 = torch.Generator().manual_seed(6)
     prompts = [torch.randint(0, 71, (n,), generator=g2).tolist() for n in (9, 1, 23, 14)]
     for policy in ("reserve_full", "optimistic"):
+        # (the second time with every decode step size recorded before the first request: three requests
+        # at most, no pages: the sizes 1, 2 and 4)
+        at_start = policy == "optimistic"
         llm = LLM(mdir, dtype="float32", num_blocks=4, block_size=16, max_batch_size=3, chunk_size=8, max_num_batched_tokens=16,
-                  enable_graph=True, admission=policy)
+                  enable_graph=True, admission=policy, record_graphs_at_start=at_start)
         assert not llm.engine.runner.cache.groups
+        assert len(llm.engine.runner._graphs) == (3 if at_start else 0)
         outs = llm.generate(prompt_token_ids=prompts, sampling_params=SamplingParams(top_k=1, max_tokens=12, ignore_eos=True))
         for p, o in zip(prompts, outs):
             assert o.outputs[0].token_ids == plain_greedy(p, 12), f"{policy}: prompt of {len(p)} tokens"
         assert llm.engine.runner._graphs, "no decode step was recorded"
+        assert not at_start or len(llm.engine.runner._graphs) == 3
         llm.engine.runner.cache.check()
         llm.close()
