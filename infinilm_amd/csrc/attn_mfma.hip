@@ -862,17 +862,6 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
 
 extern "C" int ilm_attn_tile_tokens() { return ATT_TT; }
 
-static int att_num_cus() {
-    static int n = 0;
-    if (n == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
-        if (n <= 0) n = 256;
-    }
-    return n;
-}
-
 extern "C" int ilm_attn_tile(void* out, const void* q, const void* kc, const void* vc, const void* block_tables,
                              const void* seg, const void* pos, const void* tiles, int n_tiles, int nh, int nkv,
                              int d, int page, int max_blocks, int q_stride, int out_stride, float scale,
@@ -886,7 +875,7 @@ extern "C" int ilm_attn_tile(void* out, const void* q, const void* kc, const voi
     ILM_REQUIRE(nkv * HG <= 65535, "attn_tile: grid too large");
     dim3 grid(n_tiles, nkv * HG);
     const float sl2 = scale * 1.4426950408889634f;
-    const int cus = att_num_cus();
+    const int cus = ilm_num_cus();
     const long long n_items = (long long)n_tiles * nkv * HG;
     const int pair_base = (n_items > cus && n_items <= 2 * cus) ? cus : 0;
 #define AT_ARGS (bf16*)out, (const bf16*)q, (const bf16*)kc, (const bf16*)vc, (const int*)block_tables, (const int*)seg, \

@@ -81,6 +81,8 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 
 extern "C" const char* ilm_last_error();
 void ilm_set_error(const char* fmt, ...);
+// compute units of the current device (looked up once a process; 256 if the runtime does not say)
+int ilm_num_cus();
 
 #define ILM_REQUIRE(cond, ...)          \
     do {                                \

@@ -15,6 +15,17 @@ void ilm_set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
+int ilm_num_cus() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
 // ------------------------------------------------------------------------------------------
 // embedding: r[t, :] = scale * E[ids[t], :]   (residual stream, float)
 // ------------------------------------------------------------------------------------------

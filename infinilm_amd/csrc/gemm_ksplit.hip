@@ -136,17 +136,6 @@ gemm_ksplit_kernel(TC* __restrict__ C, const bf16* __restrict__ X, const bf16* _
     }
 }
 
-static int gf_num_cus() {
-    static int n = 0;
-    if (n == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
-        if (n <= 0) n = 256;
-    }
-    return n;
-}
-
 // Largest K a call takes, given how many parts the caller lets the result be split into.
 extern "C" int ilm_gemm_ksplit_max_k(int parts) { return GF_KSPAN * parts; }
 
@@ -164,7 +153,7 @@ extern "C" int ilm_gemm_ksplit(void* C, int out_dtype, int ldc, long c_part_stri
                 "gemm_ksplit: X and W rows must be 16-byte aligned, X rows %d long", act ? 2 * K : K);
     const int ntiles = (N + 15) / 16;
     const int kspan = ((K + kb - 1) / kb + 31) / 32 * 32;   // K spread evenly over the parts
-    int gx = gf_num_cus() / kb;
+    int gx = ilm_num_cus() / kb;
     if (gx < 1) gx = 1;
     if (gx > ntiles) gx = ntiles;
     dim3 grid(gx, kb);

@@ -147,17 +147,6 @@ gemm_qkv_rope_kernel(bf16* __restrict__ Q, const bf16* __restrict__ X, const bf1
     }
 }
 
-static int qr_num_cus() {
-    static int n = 0;
-    if (n == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
-        if (n <= 0) n = 256;
-    }
-    return n;
-}
-
 // Q [M, ldq] receives the rotated query heads; k (rotated) and v go to the cache slots (slots may be
 // null: nothing is cached).  W [(nh + 2 nkv) d, ldw] holds the q, k, v rows in this order.
 extern "C" int ilm_gemm_qkv_rope(void* Q, int ldq, const void* X, int lda, const void* W, int ldw, const void* bias,
@@ -175,7 +164,7 @@ extern "C" int ilm_gemm_qkv_rope(void* Q, int ldq, const void* X, int lda, const
     const int total_pairs = (nh + 2 * nkv) * (d / 2);
 #define QR_CASE(WV, KS, MGR)                                                                                   \
     {                                                                                                          \
-        const int cap = qr_num_cus() * ((WV == 16 || (MGR == 2 && KS >= 12)) ? 1 : 2);                         \
+        const int cap = ilm_num_cus() * ((WV == 16 || (MGR == 2 && KS >= 12)) ? 1 : 2);                         \
         int ppu = (total_pairs + cap - 1) / cap;                                                               \
         if (ppu > 16) ppu = 16;                                                                                \
         const int n_units = (total_pairs + ppu - 1) / ppu;                                                     \

@@ -118,17 +118,6 @@ gemm_rows64_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16
     }
 }
 
-static int r6_num_cus() {
-    static int n = 0;
-    if (n == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
-        if (n <= 0) n = 256;
-    }
-    return n;
-}
-
 extern "C" int ilm_gemm_rows64_span() { return R6_SPAN; }
 
 // C: float [kb][M][ldc] with c_part_stride elements between the parts, kb = ceil(K / ilm_gemm_rows64_span()).
@@ -142,7 +131,7 @@ extern "C" int ilm_gemm_rows64(void* C, int ldc, long c_part_stride, int kb, con
                 (K + R6_SPAN - 1) / R6_SPAN, kb);
     const int ntiles = (N + 15) / 16;
     const int n_groups = (ntiles + R6_T - 1) / R6_T;
-    int gx = r6_num_cus() / kb;
+    int gx = ilm_num_cus() / kb;
     if (gx < 1) gx = 1;
     if (gx > n_groups) gx = n_groups;
     dim3 grid(gx, kb);

@@ -450,19 +450,6 @@ gemm_gateup_swiglu_pair_kernel(bf16* __restrict__ C, const bf16* __restrict__ X,
     }
 }
 
-static int g_num_cus = 0;
-
-static int num_cus() {
-    if (g_num_cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            g_num_cus = prop.multiProcessorCount;
-        if (g_num_cus <= 0) g_num_cus = 256;
-    }
-    return g_num_cus;
-}
-
 // variant: 0 = choose; 4 = resident; 1, 2, 3, 5, 6 = shapes of the stream kernel (see below)
 extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void* bias, int M, int N,
                                int K, int lda, int ldw, int ldc, float alpha, int out_dtype, int variant,
@@ -485,7 +472,7 @@ extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void
         const int ntiles = (N + 15) / 16;
 #define SR_CASE(WV, KS, MGR, PER_CU, TC)                                                                    \
     {                                                                                                       \
-        const int grid = ntiles < num_cus() * PER_CU ? ntiles : num_cus() * PER_CU;                         \
+        const int grid = ntiles < ilm_num_cus() * PER_CU ? ntiles : ilm_num_cus() * PER_CU;                         \
         gemm_skinny_resident_kernel<WV, KS, MGR, TC><<<grid, WV * 64, 0, stream>>>(                         \
             (TC*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, lda, ldw, ldc, alpha, ntiles, \
             (ksteps + WV - 1) / WV);                                                                        \
@@ -496,7 +483,7 @@ extern "C" int ilm_gemm_skinny(void* C, const void* X, const void* W, const void
         // (q/k/v).  Two tiles in flight instead of one changed nothing.  INFINILM_AMD_SKINNY_FAT=0: always 16 x 8.
         static int fat = -1;
         if (fat < 0) { const char* e = getenv("INFINILM_AMD_SKINNY_FAT"); fat = e ? atoi(e) : 1; }
-        const bool fat_waves = fat && ksteps > 8 * 8 && ksteps <= 8 * 16 && (ntiles <= num_cus() || ntiles >= 4 * num_cus());
+        const bool fat_waves = fat && ksteps > 8 * 8 && ksteps <= 8 * 16 && (ntiles <= ilm_num_cus() || ntiles >= 4 * ilm_num_cus());
 #define SR_DISPATCH(TC)                                         \
     if (mg == 2) {                                              \
         if (ksteps <= 8 * 4) SR_CASE(8, 4, 2, 2, TC)            \
@@ -565,11 +552,11 @@ extern "C" int ilm_gemm_gateup_swiglu(void* C, int ldc, const void* X, int lda, 
     const int ksteps = (K + 31) / 32;
     ILM_REQUIRE(ksteps <= (M <= 16 ? 16 * 16 : 8 * 16), "gemm_gateup_swiglu: K=%d is beyond %d", K, M <= 16 ? 8192 : 4096);
     // whole tiles in pairs where every workgroup gets at least two pairs, else tiles of 8 + 8 rows
-    const bool pairs = (I + 15) / 16 >= 2 * num_cus();
+    const bool pairs = (I + 15) / 16 >= 2 * ilm_num_cus();
     const int ntiles = pairs ? (I + 15) / 16 : (I + 7) / 8;
 #define GU_LAUNCH(KERNEL, WV, KS, MGR, PER_CU)                                                              \
     {                                                                                                       \
-        const int grid = ntiles < num_cus() * PER_CU ? ntiles : num_cus() * PER_CU;                         \
+        const int grid = ntiles < ilm_num_cus() * PER_CU ? ntiles : ilm_num_cus() * PER_CU;                         \
         KERNEL<WV, KS, MGR><<<grid, WV * 64, 0, stream>>>(                                                  \
             (bf16*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, I, K, lda, ldw, ldc, ntiles,    \
             (ksteps + WV - 1) / WV, (const float*)ss, ss_tiles, eps);                                       \

@@ -126,17 +126,6 @@ gemm_tail_kernel(float* __restrict__ R, bf16* __restrict__ XW, float* __restrict
     }
 }
 
-static int gt_num_cus() {
-    static int n = 0;
-    if (n == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
-        if (n <= 0) n = 256;
-    }
-    return n;
-}
-
 extern "C" int ilm_gemm_tail_ss_rows() { return GT_SS_ROWS; }
 
 // R [M, ldr] float in/out; XW [M, ldxw] bfloat16 out; SS [ceil(N / 16), ilm_gemm_tail_ss_rows()] float out (rows
@@ -155,7 +144,7 @@ extern "C" int ilm_gemm_tail(void* R, int ldr, void* XW, int ldxw, void* SS, con
     const int ntiles = (N + 15) / 16;
 #define GT_LAUNCH(WV, KS, MGR, PER_CU, NWT)                                                                       \
     {                                                                                                             \
-        const int grid = ntiles < gt_num_cus() * PER_CU ? ntiles : gt_num_cus() * PER_CU;                         \
+        const int grid = ntiles < ilm_num_cus() * PER_CU ? ntiles : ilm_num_cus() * PER_CU;                         \
         gemm_tail_kernel<WV, KS, MGR, NWT><<<grid, WV * 64, 0, stream>>>(                                         \
             (float*)R, (bf16*)XW, (float*)SS, (const bf16*)X, (const bf16*)W, (const bf16*)bias, (const NWT*)norm_w, \
             M, N, K, lda, ldw, ldr, ldxw, alpha, ntiles, (ksteps + WV - 1) / WV);                                 \
