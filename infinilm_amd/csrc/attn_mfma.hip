@@ -374,7 +374,8 @@ attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, cons
 // ------------------------------------------------------------------------------------------------
 // Tiles of up to ATT_TT consecutive tokens of one request (portions of prompts): the 4 waves of a
 // workgroup take 2 tokens each and share every 64-key tile of K and V through LDS (the next tile is
-// already on its way into registers), so a tile is read from the cache once per 8 tokens x 16 heads.  No key chunks and no
+// already on its way: into registers, or, for heads of 128 and pages that hold whole tiles, straight
+// into a second pair of LDS buffers), so a tile is read from the cache once per 8 tokens x 16 heads.  No key chunks and no
 // workspace: one workgroup walks all keys its tokens see, in ascending order of absolute key
 // index, 32 at a time.
 // ------------------------------------------------------------------------------------------------
@@ -402,8 +403,18 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     constexpr bool SWZ = D == 128;
     constexpr int KROW = SWZ ? D : D + 8;
     constexpr int VROW = SWZ ? ATT_TK : ATT_TK + 8;
-    __shared__ __attribute__((aligned(16))) bf16 Ks[ATT_TK * KROW];
-    __shared__ __attribute__((aligned(16))) bf16 Vs[D * VROW];
+    // DIRECT (head size 128 and pages that hold whole tiles): a tile goes from the cache into LDS without passing
+    // through registers (global_load_lds_dwordx4: lane l's 16 bytes land at the instruction's LDS base + 16 l, so
+    // the exchange of a row's pieces is made on the source side: the lane that fills a slot reads the piece
+    // that belongs there).  The loads of the next tile are then on their way into a second pair of buffers
+    // while this one is multiplied, with one barrier a tile and no stores to LDS.  Measured at 2,048 tokens: of
+    // 63 us a layer, 8 were the loads into registers and 6 the stores into LDS (timing runs without them).
+    constexpr bool DIRECT = SWZ && PAGE64;
+    constexpr int NBUF = DIRECT ? 2 : 1;
+    __shared__ __attribute__((aligned(16))) bf16 Ks2[NBUF][ATT_TK * KROW];
+    __shared__ __attribute__((aligned(16))) bf16 Vs2[NBUF][D * VROW];
+    const bf16* Ks = Ks2[0];   // the tile being multiplied
+    const bf16* Vs = Vs2[0];
     auto k_at = [](int row, int piece) -> int { return row * KROW + (SWZ ? (piece ^ (row & 15)) : piece) * 8; };
     auto v_at = [](int row, int piece) -> int { return row * VROW + (SWZ ? (piece ^ ((row >> 1) & 7)) : piece) * 8; };
     __shared__ int bt_s[ATT_BT_LDS];
@@ -516,13 +527,37 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
         // consecutive rows, which the row padding spreads over all banks.
         const int kk = pc / (D / 8);
         const int prow = (kk & 32) | ((kk & 4) << 2) | ((kk & 24) >> 1) | (kk & 3);
-        if (pc < KPIECES) *reinterpret_cast<uint4*>(&Ks[k_at(prow, pc % (D / 8))]) = v;
+        if (pc < KPIECES) *reinterpret_cast<uint4*>(&Ks2[0][k_at(prow, pc % (D / 8))]) = v;
     };
     auto stash_v = [&](int i, uint4 v) {
         const int pc = tid + i * 256;
-        if (pc < VPIECES) *reinterpret_cast<uint4*>(&Vs[v_at(v_row(pc), pc % (ATT_TK / 8))]) = v;
+        if (pc < VPIECES) *reinterpret_cast<uint4*>(&Vs2[0][v_at(v_row(pc), pc % (ATT_TK / 8))]) = v;
     };
     uint4 k0 = zero4, k1 = zero4, k2 = zero4, k3 = zero4, v0 = zero4, v1 = zero4, v2 = zero4, v3 = zero4;
+    // DIRECT: instruction u of this wave fills the 64 consecutive 16-byte slots from (wave * 4 + u) * 64 on, of K and
+    // of V; this lane's slot of it holds, K: piece (slot & 15) ^ (row & 15) of the key whose row it is (the inverse
+    // of stash_k's row order), V: keys ((slot & 7) ^ ((row >> 1) & 7)) * 8 .. + 8 of dim row = slot >> 3
+    int kdir[4], vdir[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int i = (wave * 4 + u) * 64 + lane;
+        const int krow = i >> 4, kslot = i & 15;
+        const int key = (krow & 32) | ((krow & 16) >> 2) | ((krow & 12) << 1) | (krow & 3);
+        kdir[u] = key * D + ((kslot ^ (krow & 15)) * 8);
+        const int vrow = i >> 3, vslot = i & 7;
+        vdir[u] = vrow * page + ((vslot ^ ((vrow >> 1) & 7)) * 8);
+    }
+    typedef __attribute__((address_space(3))) void* lds_ptr;
+#define ATT_FETCH_DIRECT(kb_, BUF_)                                                                            \
+    {                                                                                                          \
+        const int pg_ = page_of(kb_);                                                                          \
+        const bf16* kt_ = kc + (((size_t)pg_ * nkv + kvh) * page + ((kb_) % page)) * D;                        \
+        const bf16* vt_ = vc + ((size_t)pg_ * nkv + kvh) * D * page + ((kb_) % page);                          \
+        _Pragma("unroll") for (int u = 0; u < 4; ++u)                                                          \
+            __builtin_amdgcn_global_load_lds((const void*)(kt_ + kdir[u]), (lds_ptr)(&Ks2[BUF_][(wave * 4 + u) * 512]), 16, 0, 0); \
+        _Pragma("unroll") for (int u = 0; u < 4; ++u)                                                          \
+            __builtin_amdgcn_global_load_lds((const void*)(vt_ + vdir[u]), (lds_ptr)(&Vs2[BUF_][(wave * 4 + u) * 512]), 16, 0, 0); \
+    }
 #define ATT_FETCH(kb_)                          \
     if (PAGE64) {                               \
         const int pg_ = page_of(kb_);           \
@@ -549,12 +584,30 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
 
     const int kb0 = lo_first & ~(ATT_TK - 1);
     __syncthreads();   // bt_s is filled
-    ATT_FETCH(kb0)
-    // every tile begins with the exchange of the staged registers for the tile in LDS
-    auto tile_begin = [&]() {
-        __syncthreads();   // the previous tile has been consumed
-        ATT_STASH()
-        __syncthreads();
+    int cur = 0;       // DIRECT: the buffers of the tile that is multiplied next
+    if (DIRECT) {
+        ATT_FETCH_DIRECT(kb0, 0)
+    } else {
+        ATT_FETCH(kb0)
+    }
+    // every tile begins with the exchange of the staged registers for the tile in LDS; DIRECT: with the wait
+    // for this tile's loads, after which (and a barrier: everybody's have landed, and everybody is done with the
+    // tile before) the loads of the next tile go into the other buffers
+    auto tile_begin = [&](int kb) {
+        if (DIRECT) {
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            Ks = Ks2[cur];
+            Vs = Vs2[cur];
+            cur ^= 1;
+            if (kb + ATT_TK <= p_last) {
+                if (cur) ATT_FETCH_DIRECT(kb + ATT_TK, 1) else ATT_FETCH_DIRECT(kb + ATT_TK, 0)
+            }
+        } else {
+            __syncthreads();   // the previous tile has been consumed
+            ATT_STASH()
+            __syncthreads();
+        }
     };
     // A tile that both tokens of the wave see whole (every tile but those on the diagonal and at a
     // window's edge) takes a path without masks, written so that matrix and vector instructions
@@ -646,7 +699,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
             __builtin_amdgcn_sched_barrier(0);
         }
         // the next tile leaves for the registers only now: until here they held score fragments
-        if (kb + ATT_TK <= p_last) { ATT_FETCH(kb + ATT_TK) }
+        if (!DIRECT && kb + ATT_TK <= p_last) { ATT_FETCH(kb + ATT_TK) }
         // values of the first sub-tile; their products stand between the p of the second
         // (should the reference point move now, the first sub-tile's products, made with the old one,
         // are added first, and the interleaved block below adds zeros in their place)
@@ -712,7 +765,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     };
     // any tile: masks where a token does not see a key
     auto general_tile = [&](int kb) {
-        if (kb + ATT_TK <= p_last) { ATT_FETCH(kb + ATT_TK) }   // in flight while this tile is multiplied
+        if (!DIRECT && kb + ATT_TK <= p_last) { ATT_FETCH(kb + ATT_TK) }   // in flight while this tile is multiplied
         // The score products of both 32-key sub-tiles are issued first, so that the matrix cores
         // work on the second while the vector units do the softmax of the first.
         constexpr int NSUB = ATT_TK / 32;
@@ -830,15 +883,15 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     if (D % 32 != 0 || kb_b < kb_a) kb_a = kb_b = kb0;
     int kb = kb0;
     for (; kb < kb_a && kb <= p_last; kb += ATT_TK) {
-        tile_begin();
+        tile_begin(kb);
         general_tile(kb);
     }
     for (; kb < kb_b; kb += ATT_TK) {
-        tile_begin();
+        tile_begin(kb);
         fast_tile(kb);
     }
     for (; kb <= p_last; kb += ATT_TK) {
-        tile_begin();
+        tile_begin(kb);
         general_tile(kb);
     }
     if (!head_ok) return;
@@ -858,6 +911,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
 }
 
 #undef ATT_FETCH
+#undef ATT_FETCH_DIRECT
 #undef ATT_STASH
 
 extern "C" int ilm_attn_tile_tokens() { return ATT_TT; }
