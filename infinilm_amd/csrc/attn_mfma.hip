@@ -1036,6 +1036,11 @@ static int scratch_of_current_device(float** ptr) {
 
 extern "C" long ilm_attn_static_scratch_floats() { return (long)ILM_ATTN_SCRATCH_FLOATS; }
 
+extern "C" int ilm_attn_static_init() {
+    float* base = nullptr;
+    return scratch_of_current_device(&base);
+}
+
 extern "C" int ilm_attn_mfma_static(void* out, const void* q, const void* kc, const void* vc,
                                     const void* block_tables, const void* seg, const void* pos, const void* rows,
                                     int T_, int nh, int nkv, int d, int page, int max_blocks, int q_stride,

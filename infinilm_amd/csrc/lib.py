@@ -76,6 +76,8 @@ def load(verbose: bool = True) -> ctypes.CDLL:
                                "(python -c 'import __graft_entry__ as g; g.build()')")
         fn.argtypes = args
         fn.restype = c_int
+    lib.ilm_attn_static_init.restype = c_int
+    lib.ilm_attn_static_init.argtypes = []
     lib.ilm_attn_static_scratch_floats.restype = c_long
     lib.ilm_attn_static_scratch_floats.argtypes = []
     _lib = lib

@@ -17,8 +17,10 @@ extern "C" {
 // scratch.  Needs T * nh * nsplit * (d + 2) <= ILM_ATTN_SCRATCH_FLOATS floats (64 tokens x 32 heads x
 // 16 chunks x 130 at most, for instance); beyond that it returns -1 with a message and launches
 // nothing.  With nsplit == 1 the scratch is not used.  It calls no hipMalloc, hipFree or other
-// allocating routine; the scratch's address is looked up once per device, at the first call with
-// that device current.  Every slot the merge kernel reads is written by the attention kernel of the
+// allocating routine; the scratch's address is looked up once per device: by ilm_attn_static_init(), or
+// else at the first call with that device current (a caller that records HIP graphs calls
+// ilm_attn_static_init() before its first capture on a device, so that the look-up, which is no stream
+// operation, does not fall into a capture).  Every slot the merge kernel reads is written by the attention kernel of the
 // same call, so nothing has to be cleared between calls.  All calls on one GPU share that GPU's
 // scratch: calls that overlap on one GPU (two streams, two threads) race; calls on one stream are
 // ordered and safe.  Arguments, results and return value otherwise as ilm_attn_mfma.
@@ -26,6 +28,10 @@ int ilm_attn_mfma_static(void* out, const void* q, const void* kc, const void* v
                          const void* seg, const void* pos, const void* rows, int T, int nh, int nkv, int d,
                          int page, int max_blocks, int q_stride, int out_stride, float scale, int window,
                          int nsplit, int span, hipStream_t stream);
+
+// Looks up the scratch's address on the current device (once; later calls return at once).  0, or -1
+// with a message.  Allocates nothing.
+int ilm_attn_static_init();
 
 // ILM_ATTN_SCRATCH_FLOATS, for callers that size their calls at run time.
 long ilm_attn_static_scratch_floats();

@@ -15,6 +15,7 @@ pairing).  The arithmetic is the tensor library's in the reference; the definiti
 """
 from __future__ import annotations
 
+import inspect
 import math
 from typing import Callable, Dict, Optional, Tuple
 
@@ -24,7 +25,7 @@ from .. import kernels
 from .base import BuildContext, PositionEncoding
 from .registry import register_position_encoding
 
-# kind -> function(inv_freq float64 [rd/2], params, max_positions) -> (inv_freq, magnitude)
+# kind -> function(inv_freq float64 [rd/2], params, max_positions[, theta=base]) -> (inv_freq, magnitude)
 SCALINGS: Dict[str, Callable] = {}
 
 
@@ -126,9 +127,16 @@ class RotaryEmbedding(PositionEncoding):
             if kind not in SCALINGS:
                 raise ValueError(f"Unsupported rope_scaling_type: {kind}")
             fn = SCALINGS[kind]
-            # a scaling that takes a fourth argument is given the base theta (yarn's band edges need it)
-            if fn.__code__.co_argcount >= 4:
-                inv_freq, m = fn(inv_freq, self.scaling, self.max_positions, self.theta)
+            # a scaling that names a `theta` parameter (or takes any keyword) is given the base theta by
+            # keyword (yarn's band edges need it); the signature is looked at, not the code object, so
+            # partials and wrapped callables work too
+            try:
+                params = inspect.signature(fn).parameters
+                takes_theta = "theta" in params or any(p.kind is p.VAR_KEYWORD for p in params.values())
+            except (TypeError, ValueError):
+                takes_theta = False
+            if takes_theta:
+                inv_freq, m = fn(inv_freq, self.scaling, self.max_positions, theta=self.theta)
             else:
                 inv_freq, m = fn(inv_freq, self.scaling, self.max_positions)
         p = torch.arange(self.max_positions, dtype=torch.float64)

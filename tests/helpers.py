@@ -12,7 +12,7 @@ import torch
 
 import plain_minicpm4 as P
 
-CONFIGS = {"A": P.tiny_config_a, "B": P.tiny_config_b, "C": P.tiny_config_c}
+CONFIGS = {"A": P.tiny_config_a, "B": P.tiny_config_b, "C": P.tiny_config_c, "D": P.tiny_config_d, "E": P.tiny_config_e}
 
 
 def make_model_dir(path: str, cfg: dict, seed: int, store: str = "float32", sharp: bool = True):

@@ -117,11 +117,67 @@ def plain_rope_tables(cfg: dict):
                 s = max_pos / orig
             if s > 1.0:
                 m = math.sqrt(1.0 + math.log(s) / math.log(orig))
+        elif kind == "llama3":
+            inv_freq = torch.tensor(plain_llama3_frequencies(inv_freq.tolist(), rs), dtype=DT)
+        elif kind == "yarn":
+            freqs, m = plain_yarn_frequencies(inv_freq.tolist(), rs, rd, theta)
+            inv_freq = torch.tensor(freqs, dtype=DT)
         else:
             raise ValueError("Unsupported rope_scaling_type: " + str(kind))
     p = torch.arange(max_pos, dtype=DT)
     ang = p[:, None] * inv_freq[None, :]
     return torch.cos(ang) * m, torch.sin(ang) * m
+
+
+def plain_llama3_frequencies(inv_freq: Sequence[float], rs: dict) -> list:
+    """`llama3` scaling, pair by pair.  Keys (all required): factor, low_freq_factor, high_freq_factor,
+    original_max_position_embeddings: rope_scaling_creators.cpp:54-75.  The arithmetic is not in the
+    reference's text (it lies in its tensor library): parity unpinned.  Definition used: a pair that
+    turns more than high_freq_factor times within the original length keeps its frequency; one that turns
+    less than low_freq_factor times has it divided by factor; between the two the division is blended in
+    linearly in the number of turns."""
+    factor, low, high = float(rs["factor"]), float(rs["low_freq_factor"]), float(rs["high_freq_factor"])
+    orig = float(rs["original_max_position_embeddings"])
+    out = []
+    for w in inv_freq:
+        turns = orig * w / (2.0 * math.pi)     # full turns of this pair over the original length
+        if turns > high:
+            out.append(w)
+        elif turns < low:
+            out.append(w / factor)
+        else:
+            t = (turns - low) / (high - low)
+            out.append(t * w + (1.0 - t) * w / factor)
+    return out
+
+
+def plain_yarn_frequencies(inv_freq: Sequence[float], rs: dict, rd: int, theta: float):
+    """`yarn` scaling, pair by pair; returns (frequencies, magnitude of cos and sin).  Keys and defaults:
+    factor and original_max_position_embeddings required, beta_fast 32, beta_slow 1 (cut to whole numbers),
+    mscale 1, mscale_all_dim 0, the rotary dim and rope_theta from the model: rope_scaling_creators.cpp:80-102.
+    The arithmetic is not in the reference's text: parity unpinned.  Definition used: the pair index at
+    which a pair turns beta times within the original length is rd * ln(orig / (2 pi beta)) / (2 ln theta);
+    pairs below the index for beta_fast (rounded down, at least 0) keep their frequency, pairs above the
+    index for beta_slow (rounded up, at most the last pair) have it divided by factor, a linear ramp
+    between; the magnitude is (0.1 mscale ln factor + 1) / (0.1 mscale_all_dim ln factor + 1) for factor > 1."""
+    factor, orig = float(rs["factor"]), float(rs["original_max_position_embeddings"])
+    beta_fast, beta_slow = int(rs.get("beta_fast", 32)), int(rs.get("beta_slow", 1))
+
+    def index_of(beta):
+        return rd * math.log(orig / (2.0 * math.pi * beta)) / (2.0 * math.log(theta))
+
+    first = max(math.floor(index_of(beta_fast)), 0)
+    last = min(math.ceil(index_of(beta_slow)), rd // 2 - 1)
+    width = max(last - first, 0.001)
+    out = []
+    for i, w in enumerate(inv_freq):
+        stretched = min(max((i - first) / width, 0.0), 1.0)   # 0: kept, 1: divided by factor
+        out.append(w * (1.0 - stretched) + (w / factor) * stretched)
+
+    def gain(mscale):
+        return 0.1 * mscale * math.log(factor) + 1.0 if factor > 1.0 else 1.0
+
+    return out, gain(float(rs.get("mscale", 1.0))) / gain(float(rs.get("mscale_all_dim", 0.0)))
 
 
 def plain_apply_rope(x: torch.Tensor, pos: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
@@ -366,6 +422,33 @@ def tiny_config_c() -> dict:
         "scale_emb": 7, "scale_depth": 2.0, "tie_word_embeddings": True,
         "rope_scaling": {"rope_type": "longrope", "short_factor": short, "long_factor": long,
                          "original_max_position_embeddings": 512},
+    }
+
+
+def tiny_config_d() -> dict:
+    """`llama3` scaling whose three bands (kept, blended, divided) all hold pairs of a head of 32; every
+    head its own keys."""
+    return {
+        "architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm4", "torch_dtype": "float32",
+        "num_hidden_layers": 2, "hidden_size": 72, "num_attention_heads": 3,
+        "num_key_value_heads": 3, "head_dim": 32, "intermediate_size": 136, "vocab_size": 211,
+        "rope_theta": 10000.0, "max_position_embeddings": 320, "rms_norm_eps": 2e-6,
+        "scale_emb": 3, "scale_depth": 1.2, "dim_model_base": 36, "tie_word_embeddings": False,
+        "rope_scaling": {"rope_type": "llama3", "factor": 6.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                         "original_max_position_embeddings": 64},
+    }
+
+
+def tiny_config_e() -> dict:
+    """`yarn` scaling with a ramp over the middle pairs of a head of 64 and a magnitude other than 1."""
+    return {
+        "architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm", "torch_dtype": "float32",
+        "num_hidden_layers": 2, "hidden_size": 88, "num_attention_heads": 4,
+        "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 152, "vocab_size": 173,
+        "rope_theta": 5000.0, "max_position_embeddings": 384, "rms_norm_eps": 1e-5,
+        "scale_emb": 5, "scale_depth": 1.6, "tie_word_embeddings": True,
+        "rope_scaling": {"type": "yarn", "factor": 6.0, "original_max_position_embeddings": 64, "beta_fast": 8,
+                         "beta_slow": 1, "mscale": 0.8, "mscale_all_dim": 0.3},
     }
 
 

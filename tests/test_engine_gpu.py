@@ -678,3 +678,130 @@ def test_layers_of_real_size_against_the_plain_implementation(shape):
     print(f"[err] real size {shape}: float32 {err32:.3e}, bfloat16 {err16:.3e}")
     assert err32 < 1e-4, f"float32 against the plain implementation at real size: {err32:.3e}"
     assert err16 < TOL["bfloat16"], f"bfloat16 against the plain implementation at real size: {err16:.3e}"
+
+
+def _both_dtypes(cfg, num_pages, _unused=None):
+    """Builds the configuration's model with the same (bfloat16-representable) random weights in float32 (eager
+    steps) and in bfloat16 (decode steps recorded as graphs) and yields (dtype, runner, weights for the plain implementation) for each."""
+    from infinilm_amd.engine.loading import build_model, make_runner
+    from infinilm_amd.weights import fill_random_
+
+    tied = bool(cfg.get("tie_word_embeddings"))
+    for dtype, graph in (("float32", False), ("bfloat16", True)):
+        model = build_model(cfg, dtype, "cuda:0")
+        fill_random_(model, seed=1, std=0.02, norm_init="one_plus", tie=tied)
+        if dtype == "float32":   # the same values the bfloat16 model holds
+            for p in model.named_parameters().values():
+                p.tensor.copy_(p.tensor.to(torch.bfloat16).to(torch.float32))
+        r = make_runner(model, num_pages=num_pages, page_size=64, max_requests=4, enable_graph=graph)
+        W = {n: p.tensor for n, p in model.named_parameters().items() if not (tied and n == "lm_head.weight")}
+        yield dtype, r, W
+        del r, model, W
+        torch.cuda.empty_cache()
+
+
+def test_mixed_steps_at_the_8b_head_shape_with_recorded_steps_and_pages_used_again():
+    """Two layers of the 8B shape (heads of 128 in groups of 16, pages of 64): five requests over a pool of 13
+    pages, up to four live.  One step holds a portion with history, two decoded tokens and a fresh prompt
+    (the tile attention's direct loads beside the chunked kernel, the library's products); one holds
+    the same mix in 12 rows (the few-rows products with rotation, cache write, residual sum and half a norm in
+    their epilogues); the steps of four decoded tokens replay a recording in bfloat16; the last request gets
+    pages that two finished ones gave back.  Every logit of every request against the plain implementation
+    in float64, in 32-bit and in bfloat16."""
+    from infinilm_amd.engine.step import StepEntry
+
+    cfg = _real_shape("8b")
+    g = torch.Generator().manual_seed(11)
+    lens = {"a": 340, "b": 140, "c": 70, "d": 150, "e": 100}
+    toks = {r: torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for r, n in lens.items()}
+    steps = [([("b", 130), ("c", 60)], []),
+             ([("a", 200), ("b", 1), ("c", 1)], []),
+             ([("a", 90), ("b", 1), ("c", 1), ("d", 140)], [])]        # a portion with history, two decoded tokens, a fresh prompt
+    steps += [([("a", 1), ("b", 1), ("c", 1), ("d", 1)], [])] * 7
+    steps += [([("a", 1), ("b", 1), ("c", 1), ("d", 1)], ["b", "c"])]
+    steps += [([("a", 5), ("d", 1), ("e", 6)], []),                     # the same mix in 12 rows
+              ([("a", 1), ("d", 1), ("e", 60)], ["d"]),
+              ([("a", 36), ("e", 1)], ["a"]),
+              ([("e", 2)], [])]
+    steps += [([("e", 1)], [])] * 31
+    oracle = None
+    for dtype, r, W in _both_dtypes(cfg, 13, None):
+        if oracle is None:
+            oracle = {q: P.plain_forward(cfg, W, t).cpu() for q, t in toks.items()}
+        fed = {q: 0 for q in toks}
+        got = {q: [] for q in toks}
+        old_pages, replays = set(), 0
+        for entries, end in steps:
+            es = []
+            for q, n in entries:
+                if not r.cache.has(q):
+                    r.cache.admit(q)
+                es.append(StepEntry(q, toks[q][fed[q]:fed[q] + n], list(range(n))))
+            before = len(r._graphs)
+            singles = all(n == 1 for _, n in entries)
+            out = r.step(es).cpu().clone()
+            replays += int(singles and r.enable_graph and len(r._graphs) == before and bool(r._graphs))
+            row = 0
+            for q, n in entries:
+                got[q].append(out[row:row + n])
+                row += n
+                fed[q] += n
+            for q in end:
+                old_pages |= set(r.cache.table(q, 0))
+                r.cache.release(q)
+            r.cache.check()
+            if entries[-1] == ("e", 6):
+                assert set(r.cache.table("e", 0)) <= old_pages, "the last request's pages were not used before"
+        assert fed == lens
+        r.cache.release("e")
+        assert r.cache.free_pages() == 13
+        if r.enable_graph:
+            assert replays >= 6, "the decode steps did not replay a recording"
+        tol = 1e-4 if dtype == "float32" else TOL["bfloat16"]
+        for q in toks:
+            err = rel_err(torch.cat(got[q]), oracle[q])
+            print(f"[err] mixed steps at the 8B head shape, {dtype}, request {q}: {err:.3e}")
+            assert err < tol, f"{dtype}, request {q}: {err:.3e}"
+
+
+def test_a_context_beyond_9000_tokens_at_the_benchmark_configuration():
+    """Two layers of the configuration the benchmark times (examples/shapes.py: 32,768 positions, LongRoPE with
+    64 factors): a prompt of 9,100 tokens in portions of 2,048, then decoded tokens, against the plain
+    implementation in float64 on the same weights: positions far beyond a page table's first entries, the
+    long tiles of the portion attention and 142 pages under one decoded token."""
+    from infinilm_amd.engine.step import StepEntry
+
+    sys.path.insert(0, os.path.join(ROOT, "examples"))
+    from shapes import shape_config
+
+    cfg = shape_config("8b", 2)
+    N = 9100
+    g = torch.Generator().manual_seed(5)
+    prompt = torch.randint(0, cfg["vocab_size"], (N,), generator=g).tolist()
+    want_rows, i = [], 0
+    while i < N - 1:
+        k = min(2048, N - 1 - i)
+        want_rows += [i, i + k // 2, i + k - 1]
+        i += k
+    want_rows += list(range(N - 1, N + 4))
+    fed, oracle = [], None
+    for dtype, r, W in _both_dtypes(cfg, N // 64 + 4, None):
+        r.cache.admit("a")
+        rows, i = [], 0
+        while i < N - 1:
+            k = min(2048, N - 1 - i)
+            rows.append(r.step([StepEntry("a", prompt[i:i + k], [0, k // 2, k - 1])]).cpu().clone())
+            i += k
+        tok = prompt[N - 1]
+        for s in range(5):
+            l = r.step([StepEntry("a", [tok], [0])]).cpu().clone()
+            rows.append(l)
+            if dtype == "float32":
+                fed.append(int(torch.argmax(l[0])))
+            tok = fed[s]   # both runs are fed the float32 run's greedy tokens
+        logits = torch.cat(rows)
+        if oracle is None:
+            oracle = P.plain_forward(cfg, W, prompt + fed[:4])[want_rows].cpu()
+        err = rel_err(logits, oracle)
+        print(f"[err] context of {N} tokens, {dtype}: {err:.3e}")
+        assert err < (1e-4 if dtype == "float32" else TOL["bfloat16"]), f"{dtype}: {err:.3e}"

@@ -111,6 +111,50 @@ def test_longrope_factor_choice_and_magnitude():
         P.plain_rope_tables(dict(cfg, rope_scaling={"type": "longrope", "short_factor": [1.0] * 16}))
 
 
+def test_llama3_and_yarn_frequency_maps():
+    """What fixes the two maps beside their stated definitions (the reference holds no arithmetic or vector
+    for them: parity unpinned): factor 1 leaves every pair alone; the fastest pair is kept and the slowest is
+    divided by the factor; the map never raises a frequency and keeps their order; the band edges fall where
+    a pair's turns within the original length cross the given numbers."""
+    rd, theta, orig = 64, 10000.0, 256
+    inv = [1.0 / theta ** (2.0 * i / rd) for i in range(rd // 2)]
+    l3 = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": orig}
+    new = P.plain_llama3_frequencies(inv, l3)
+    turns = [orig * w / (2 * math.pi) for w in inv]
+    for w, n, t in zip(inv, new, turns):
+        if t > 4.0:
+            assert n == w
+        elif t < 1.0:
+            assert n == w / 8.0
+        else:
+            assert w / 8.0 < n < w
+    assert any(1.0 <= t <= 4.0 for t in turns) and new == sorted(new, reverse=True)
+    assert P.plain_llama3_frequencies(inv, dict(l3, factor=1.0)) == pytest.approx(inv, rel=1e-15)
+    # a pair exactly on an edge belongs to both descriptions: the blend is continuous there
+    edge = 2 * math.pi * 4.0 / orig
+    assert P.plain_llama3_frequencies([edge * (1 + 1e-12)], l3)[0] == pytest.approx(P.plain_llama3_frequencies([edge * (1 - 1e-12)], l3)[0], rel=1e-9)
+
+    yn = {"factor": 4.0, "original_max_position_embeddings": orig}
+    new, m = P.plain_yarn_frequencies(inv, yn, rd, theta)
+    assert new[0] == inv[0] and new[-1] == pytest.approx(inv[-1] / 4.0) and new == sorted(new, reverse=True)
+    assert all(n <= w for n, w in zip(new, inv))
+    assert m == pytest.approx(0.1 * math.log(4.0) + 1.0)           # mscale 1 over mscale_all_dim 0
+    first = math.floor(rd * math.log(orig / (2 * math.pi * 32)) / (2 * math.log(theta)))
+    assert all(new[i] == inv[i] for i in range(max(first, 0) + 1)) and new[max(first, 0) + 1] < inv[max(first, 0) + 1]
+    same, one = P.plain_yarn_frequencies(inv, dict(yn, factor=1.0), rd, theta)
+    assert same == pytest.approx(inv, rel=1e-15) and one == 1.0
+    _, both = P.plain_yarn_frequencies(inv, dict(yn, mscale=0.7, mscale_all_dim=0.7), rd, theta)
+    assert both == pytest.approx(1.0)
+    # through the tables: the scaled configurations' scores still depend on distances only, and the yarn
+    # magnitude multiplies cos and sin alike
+    for cfg in (P.tiny_config_d(), P.tiny_config_e()):
+        cos, sin = P.plain_rope_tables(cfg)
+        mag = float(cos[0, 0])
+        assert torch.allclose(cos * cos + sin * sin, torch.full_like(cos, mag * mag))
+        assert (mag == 1.0) == (cfg["rope_scaling"].get("rope_type") == "llama3")
+        assert not torch.allclose(sin[1], P.plain_rope_tables(dict(cfg, rope_scaling=None))[1][1])
+
+
 def test_partial_rotary_dim():
     base = {"hidden_size": 64, "num_attention_heads": 2}
     assert P.plain_rotary_dim(base) == 32

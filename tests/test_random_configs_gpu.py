@@ -17,15 +17,17 @@ from helpers import TOL, Driver, random_tokens, rel_err
 
 pytestmark = pytest.mark.gpu
 
-def random_config(rng):
+def random_config(rng, wide=False):
+    """`wide`: widths from 16 and intermediate sizes from 9 on (the committed seeds keep the narrower ranges
+    their random streams were drawn with)."""
     nkv = rng.choice([1, 1, 2, 2, 3, 4])
     G = rng.choice([1, 1, 2, 2, 3, 4, 5, 8, 16, 17])
     nh = nkv * G
     d = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
     while nh * d > 2048:
         d = rng.choice([16, 32, 48, 64])
-    H = 8 * rng.randint(4, 24)
-    I = rng.choice([8 * rng.randint(4, 40), rng.randint(33, 300)])
+    H = 8 * rng.randint(2 if wide else 4, 24)
+    I = rng.choice([8 * rng.randint(2 if wide else 4, 40), rng.randint(9 if wide else 33, 300)])
     V = rng.randint(40, 700)
     max_pos = rng.choice([128, 200, 300, 520])
     cfg = {"architectures": ["MiniCPMForCausalLM"], "model_type": rng.choice(["minicpm", "minicpm4"]), "torch_dtype": "float32",
@@ -78,10 +80,11 @@ def weights(cfg, seed):
     return W
 
 
-def run_case(seed, tmp):
-    """One random configuration, one random schedule; every finished request is compared whole."""
+def run_case(seed, tmp, wide=False, tol=TOL):
+    """One random configuration, one random schedule; every finished request is compared whole.
+    Returns the worst error of the case."""
     rng = random.Random(seed)
-    cfg = random_config(rng)
+    cfg = random_config(rng, wide)
     dtype = rng.choice(["float32", "bfloat16", "bfloat16"])
     page = rng.choice([4, 8, 16, 32, 64, 128, 256])
     print(f"[case] seed {seed} {dtype} page {page} " + json.dumps({k: v for k, v in cfg.items() if k not in ("rope_scaling", "architectures")})
@@ -128,11 +131,33 @@ def run_case(seed, tmp):
             del live[r]
             err = rel_err(drv.request_logits(r, len(toks[r])), oracle[r])
             worst = max(worst, err)
-            assert err < TOL[dtype], f"seed {seed} ({dtype}, pages of {page}): request {r} of {len(toks[r])} tokens: error {err:.3e}"
+            assert err < tol[dtype], f"seed {seed} ({dtype}, pages of {page}): request {r} of {len(toks[r])} tokens: error {err:.3e}"
     assert drv.runner.cache.free_pages() == num_pages
     print(f"[ok] seed {seed} worst error {worst:.2e}", flush=True)
+    return worst
 
 
 @pytest.mark.parametrize("seed", list(range(48)))
 def test_random_configuration_and_random_steps(seed, tmp_path):
     run_case(seed, tmp_path)
+
+
+# Ten bfloat16 cases that a run of 600 further seeds of the wide generator left beyond the tolerance (4.1e-2 to
+# 6.6e-2 against 4e-2): narrow layers (intermediate sizes of 14 to 17 under widths near 100, or a width of 16 to
+# 24 under dozens of heads), where one bfloat16 rounding of an activation is a large part of a logit.
+ROUNDING_BOUND_SEEDS = [131, 144, 183, 211, 261, 267, 431, 483, 510, 633]
+
+
+@pytest.mark.parametrize("seed", ROUNDING_BOUND_SEEDS)
+def test_cases_beyond_the_tolerance_are_bound_by_rounding_not_by_a_kernel(seed, tmp_path, monkeypatch):
+    """The same case through the product kernels and through the plain kernels (the FMA product in ascending
+    k, the attention without matrix instructions, no fused epilogue): what exceeds the tolerance must exceed it
+    there too, within a factor of 1.5; a fault of a product kernel would stand out against the plain ones."""
+    from infinilm_amd import kernels
+
+    loose = {"float32": TOL["float32"], "bfloat16": 1.0}
+    product = run_case(seed, tmp_path, wide=True, tol=loose)
+    monkeypatch.setattr(kernels, "FORCE_BASIC", True)
+    plain = run_case(seed, tmp_path, wide=True, tol=loose)
+    print(f"[err] seed {seed}: product kernels {product:.3e}, plain kernels {plain:.3e}", flush=True)
+    assert product <= 1.5 * plain, f"seed {seed}: product kernels {product:.3e} against plain kernels {plain:.3e}"
