@@ -177,6 +177,13 @@ attn_basic_fold_kernel(T* __restrict__ out, const float* __restrict__ ws, const 
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    if (p / AB_CHUNK > nchunks - 1) {
+        // the caller's bound on the lengths was too small for this token: its last chunks were never computed.
+        // A row of NaNs instead of a silently wrong one.
+        T* bad = out + (size_t)t * out_stride + (size_t)h * d;
+        for (int dim = lane; dim < d; dim += 64) bad[dim] = from_f32<T>(__int_as_float(0x7fc00000));
+        return;
+    }
     float M = -INFINITY, L = 0.f;
     float ACC[4] = {0.f, 0.f, 0.f, 0.f};
     for (int c = lo / AB_CHUNK; c <= p / AB_CHUNK; ++c) {

@@ -33,6 +33,8 @@ _SIGNATURES = {
     "ilm_gemm_mid": [_P, _I, _L, _I, _I, _P, _I, _I, _I, _I, _P, _I, _I, _P],
     "ilm_gemm_qkv_rope": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "ilm_gemm_f32_skinny": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+    "ilm_gemm_f32_tile": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+    "ilm_attn_f32": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "ilm_gemm_basic": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ilm_attn_basic": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ilm_gemm_skinny": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],

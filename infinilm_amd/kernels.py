@@ -23,6 +23,9 @@ ATT_MAX_CHUNKS = 256  # most chunks a context is cut into (a wave of the merge k
 BASIC_CHUNK = 512    # keys a chunk of the plain attention kernel (ilm_attn_basic_chunk())
 BASIC_SPLIT = os.environ.get("INFINILM_AMD_BASIC_SPLIT", "1") == "1"   # 0: always one wave a (token, head)
 BASIC_SPLIT_WAVES = 4096   # (token, head) pairs up to which the plain kernel takes one wave a chunk
+F32_ATTN_CHUNK = 128   # keys a chunk of the 32-bit matrix-core attention (ilm_attn_f32_chunk())
+F32_ATTN_SPLIT = os.environ.get("INFINILM_AMD_F32_ATTN_SPLIT", "1") == "1"   # 0: always one wave a (token, head group)
+F32_ATTN_SPLIT_WAVES = 2048   # (token, head group) pairs up to which it takes one wave a chunk
 # INFINILM_AMD_BASIC=1 runs the plain kernels everywhere (for telling a kernel's fault from the engine's)
 FORCE_BASIC = os.environ.get("INFINILM_AMD_BASIC", "0") == "1"
 SKINNY_VARIANT = int(os.environ.get("INFINILM_AMD_SKINNY_VARIANT", "0"))  # 0: the kernel chooses
@@ -355,13 +358,20 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
         _run("ilm_gemm_f32_skinny", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
              w.stride(0), out.stride(0), float(alpha), _stream())
         return out
+    if (a.dtype == F32 and out_dtype == F32 and not FORCE_BASIC and F32_FEW_ROWS > 0 and K % 4 == 0 and a.stride(0) % 4 == 0
+            and w.stride(0) % 4 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        # the 32-bit path's many rows (portions of prompts): tiles on the float matrix instruction, every
+        # output summed in the few-rows kernel's order, so a row's bits do not depend on the rows around it
+        _run("ilm_gemm_f32_tile", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
+             w.stride(0), out.stride(0), float(alpha), _stream())
+        return out
     _run("ilm_gemm_basic", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0), w.stride(0),
          out.stride(0), float(alpha), _dt(a), _DT[out_dtype], _stream())
     return out
 
 
-# Rows up to which the 32-bit products take the few-rows kernel (0: always the ascending-k kernel, whose sums
-# do not depend on the number of rows at all)
+# Rows up to which the 32-bit products take the few-rows kernel; beyond, the tile kernel that sums in the same
+# order (0: neither, always the plain ascending-k kernel)
 F32_FEW_ROWS = int(os.environ.get("INFINILM_AMD_F32_FEW_ROWS", "64"))
 
 
@@ -612,10 +622,23 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
              n_single, nh, nkv, d, page, block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window),
              nsplit, span, _stream())
         return out
+    bound = block_tables.shape[1] * page if max_total_len is None else min(int(max_total_len), block_tables.shape[1] * page)
+    if (q.dtype == F32 and not FORCE_BASIC and d % 16 == 0 and d <= 256 and page % 4 == 0 and q.stride(0) % 4 == 0
+            and q.data_ptr() % 16 == 0 and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0):
+        # the 32-bit path: the group's heads side by side on the float matrix instruction.  Few tokens (decoding):
+        # one wave a chunk of keys and a fold; many: one wave a token that walks its chunks.  The same bits.
+        ws, nchunks = None, 1
+        waves = T * nkv * -(-(nh // nkv) // 16)
+        if F32_ATTN_SPLIT and waves <= F32_ATTN_SPLIT_WAVES and bound > F32_ATTN_CHUNK:
+            nchunks = -(-bound // F32_ATTN_CHUNK)
+            ws = torch.empty((T * nh * nchunks * (d + 4),), dtype=F32, device=q.device)
+        _run("ilm_attn_f32", out.data_ptr(), _ptr(ws), nchunks, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+             block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d, page,
+             block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window), _stream())
+        return out
     # The plain kernel.  Few tokens over long contexts (decoding): one wave a chunk of keys and a fold of the
     # partial results, instead of one wave a head; the bits are the same (see attn_basic.hip).
     ws, nchunks = None, 1
-    bound = block_tables.shape[1] * page if max_total_len is None else int(max_total_len)
     if BASIC_SPLIT and T * nh <= BASIC_SPLIT_WAVES and bound > BASIC_CHUNK:
         nchunks = -(-bound // BASIC_CHUNK)
         ws = torch.empty((T * nh * nchunks * (d + 2),), dtype=F32, device=q.device)

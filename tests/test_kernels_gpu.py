@@ -38,6 +38,7 @@ def test_constants_mirrored_in_python_equal_the_library(K):
     assert L.ilm_attn_tile_tokens() == K.ATT_TILE_TOKENS
     assert L.ilm_attn_mfma_step() == K.ATT_STEP
     assert L.ilm_attn_basic_chunk() == K.BASIC_CHUNK
+    assert L.ilm_attn_f32_chunk() == K.F32_ATTN_CHUNK and L.ilm_attn_f32_ws_row(128) == 132
     assert L.ilm_gemm_ksplit_max_k(1) == K.KSPLIT_SPAN
     assert L.ilm_gemm_rows64_span() == K.ROWS64_SPAN
 
@@ -177,24 +178,22 @@ def test_swiglu_and_gather(K, dtype):
 
 
 @pytest.mark.parametrize("M,N,K_", [(1, 1, 1), (5, 331, 80), (64, 96, 200), (130, 70, 33), (3, 4608, 4096), (17, 331, 4100),
-                                    (33, 50, 12296), (48, 4608, 1032), (8, 16400, 64), (20, 32768, 256), (200, 96, 200)])
+                                    (33, 50, 12296), (48, 4608, 1032), (8, 16400, 64), (20, 32768, 256), (200, 96, 200),
+                                    (65, 130, 4), (300, 1100, 1028), (129, 257, 44), (2048, 1024, 4096)])
 def test_gemm_float32_is_true_float32(K, M, N, K_):
     a, w, b = _rand((M, K_), 8), _rand((N, K_), 9), _rand((N,), 10)
     out = K.gemm(a.to(DEV), w.to(DEV), b.to(DEV), 0.25)
     want = P.plain_linear(a.to(F64), w.to(F64), b.to(F64), 0.25)
     _close(out, want, 2e-6 * math.sqrt(K_))   # no reduced-precision matrix mode: errors of float32 sums only
-    # Rows do not depend on the batch around them, bit for bit, among calls of up to 64 rows (the few-rows
-    # kernel) and among calls of more (the ascending-k kernel); between the two, by the rounding of a
-    # float32 sum in another order.
+    # Rows do not depend on the batch around them, bit for bit: the few-rows kernel (up to 64 rows) and the tile
+    # kernel (more) sum every output in one order, fixed by K alone (as does the plain ascending-k kernel, which
+    # takes every row count of a K that is no multiple of 4).
     one = K.gemm(a[M // 2:M // 2 + 1].to(DEV), w.to(DEV), b.to(DEV), 0.25)
-    if M <= 64:
-        assert torch.equal(one.cpu(), out[M // 2:M // 2 + 1].cpu())
-        some = K.gemm(a[:min(M, 3)].to(DEV), w.to(DEV), b.to(DEV), 0.25)
-        assert torch.equal(some.cpu(), out[:min(M, 3)].cpu())
-    else:
-        _close(one, out[M // 2:M // 2 + 1], 1e-6 * math.sqrt(K_))
-        more = K.gemm(torch.cat([a, a[:70]]).to(DEV), w.to(DEV), b.to(DEV), 0.25)
-        assert torch.equal(more[:M].cpu(), out.cpu())
+    assert torch.equal(one.cpu(), out[M // 2:M // 2 + 1].cpu())
+    some = K.gemm(a[:min(M, 3)].to(DEV), w.to(DEV), b.to(DEV), 0.25)
+    assert torch.equal(some.cpu(), out[:min(M, 3)].cpu())
+    more = K.gemm(torch.cat([a, a[:70]]).to(DEV), w.to(DEV), b.to(DEV), 0.25)
+    assert torch.equal(more[:M].cpu(), out.cpu())
 
 
 @pytest.mark.parametrize("M,N,K_,out_dtype", [
@@ -415,8 +414,11 @@ def _attention_case(K, dtype, nh, nkv, d, page, lens, qlens, window=0, seed=0, s
     return out, torch.cat(want)
 
 
-@pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 3, 48, 16), (5, 5, 80, 7), (2, 1, 256, 16)])
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 3, 48, 16), (5, 5, 80, 7), (2, 1, 256, 16),
+                                           (32, 2, 128, 64), (34, 2, 64, 12), (5, 1, 40, 8), (3, 3, 112, 20)])
 def test_attention_float32(K, nh, nkv, d, page):
+    """Heads in steps of 16 over pages that are multiples of 4 take the float matrix-core kernel (groups of up to
+    16 heads side by side, groups of 17 in two parts); other head and page sizes the plain kernel."""
     out, want = _attention_case(K, torch.float32, nh, nkv, d, page, lens=[1, 70, 33, 130], qlens=[1, 70, 1, 5])
     _close(out, want, 3e-6)
     out, want = _attention_case(K, torch.float32, nh, nkv, d, page, lens=[90, 20], qlens=[2, 20], window=11, seed=5)
@@ -432,11 +434,45 @@ def test_attention_float32_one_wave_a_chunk_gives_the_same_bits(K, monkeypatch):
     case = dict(lens=[1500, 700, 513, 40], qlens=[1, 1, 3, 1])
     for window in (0, 600):
         monkeypatch.setattr(K, "BASIC_SPLIT", True)
-        split, want = _attention_case(K, torch.float32, 6, 2, 48, 8, window=window, seed=4, **case)
+        split, want = _attention_case(K, torch.float32, 6, 2, 48, 7, window=window, seed=4, **case)
         monkeypatch.setattr(K, "BASIC_SPLIT", False)
-        whole, _ = _attention_case(K, torch.float32, 6, 2, 48, 8, window=window, seed=4, **case)
+        whole, _ = _attention_case(K, torch.float32, 6, 2, 48, 7, window=window, seed=4, **case)
         assert torch.equal(split.cpu(), whole.cpu())
         _close(split, want, 3e-6)
+
+
+@pytest.mark.parametrize("nh,nkv,d,page", [(6, 2, 48, 8), (32, 2, 128, 64), (17, 1, 32, 4)])
+def test_attention_float32_matrix_cores_one_wave_a_chunk_gives_the_same_bits(K, monkeypatch, nh, nkv, d, page):
+    """The float matrix-core kernel's two launch shapes agree bit for bit, with and without a window whose
+    edge falls inside a chunk, and a token gives the same bits alone as inside a batch of portions."""
+    case = dict(lens=[1500, 700, 513, 40], qlens=[1, 1, 3, 1])
+    for window in (0, 600, 100):
+        monkeypatch.setattr(K, "F32_ATTN_SPLIT", True)
+        split, want = _attention_case(K, torch.float32, nh, nkv, d, page, window=window, seed=4, **case)
+        monkeypatch.setattr(K, "F32_ATTN_SPLIT", False)
+        whole, _ = _attention_case(K, torch.float32, nh, nkv, d, page, window=window, seed=4, **case)
+        assert torch.equal(split.cpu(), whole.cpu())
+        _close(split, want, 3e-6)
+    monkeypatch.setattr(K, "F32_ATTN_SPLIT", True)
+    alone, _ = _attention_case(K, torch.float32, nh, nkv, d, page, lens=[1500], qlens=[1], seed=4)
+    among, _ = _attention_case(K, torch.float32, nh, nkv, d, page, lens=[1500, 700, 513], qlens=[40, 700, 2], seed=4)
+    assert torch.equal(alone.cpu()[0], among.cpu()[39])
+
+
+def test_attention_float32_refuses_a_bound_below_a_position_loudly(K):
+    """A caller's bound on the lengths that is too small for a token must not lose a chunk silently: the
+    fold marks the token's row with NaNs."""
+    nh, nkv, d, page = 4, 2, 32, 16
+    out, want = _attention_case(K, torch.float32, nh, nkv, d, page, lens=[700, 300], qlens=[1, 1], seed=2)
+    _close(out, want, 3e-6)
+    import infinilm_amd.kernels as kk
+    orig = kk.paged_attention
+    try:
+        kk.paged_attention = lambda *a, **kw: orig(*a, **dict(kw, max_total_len=400))
+        bad, _ = _attention_case(K, torch.float32, nh, nkv, d, page, lens=[700, 300], qlens=[1, 1], seed=2)
+    finally:
+        kk.paged_attention = orig
+    assert torch.isnan(bad[0]).all() and not torch.isnan(bad[1]).any()
 
 
 @pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 16), (3, 1, 32, 16), (6, 3, 48, 32), (32, 2, 128, 64), (16, 16, 64, 16),

@@ -4,7 +4,7 @@ changing size down to two tokens; and mixed, up to four live requests with so fe
 are used again.  In 32-bit and in bfloat16, on tiny configurations that differ in every size, and
 over page sizes from 4 to 256 tokens: bfloat16 takes the matrix-core attention kernels from pages
 of 16 on (pages of 64 and more their one-lookup-a-tile path, pages of 256 a tile that begins in the
-middle of a page), the plain attention kernel below; 32-bit always the plain one."""
+middle of a page), the plain attention kernel below; 32-bit the float matrix-core kernel."""
 import random
 
 import pytest
@@ -65,6 +65,8 @@ class _KernelsSeen:
             assert "ilm_attn_basic" not in self.calls, "bfloat16 with pages of 16 and more must not take the plain attention"
             assert not tile or self.calls.get("ilm_attn_tile", 0) > 0
             assert not single or self.calls.get("ilm_attn_mfma", 0) > 0
+        elif dtype == "float32":
+            assert self.calls.get("ilm_attn_f32", 0) > 0 and "ilm_attn_basic" not in self.calls
         else:
             assert self.calls.get("ilm_attn_basic", 0) > 0
 
