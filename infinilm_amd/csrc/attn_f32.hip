@@ -209,38 +209,47 @@ attn_f32_kernel(float* __restrict__ out, float* __restrict__ ws, const float* __
     }
 }
 
-// Folds the chunks' partial results of one (token, head) in ascending order, as the one-wave shape does.
+// Folds the chunks' partial results of one (token, head) in ascending order, as the one-wave shape does: a
+// thread a dim (the block has as many waves as the head has 64s of dims), every thread the scalars.  The
+// loads of FA_FOLD_AHEAD chunks are in flight together; the fold itself stays one chain in chunk order.
 // A token whose chunks do not all lie inside the workspace (the caller's bound was too small) gets a row of
 // NaNs instead of a silently wrong one.
-__global__ void __launch_bounds__(64)
+#define FA_FOLD_AHEAD 8
+__global__ void __launch_bounds__(256)
 attn_f32_fold_kernel(float* __restrict__ out, const float* __restrict__ ws, const int* __restrict__ pos, int nh, int d,
                      int nchunks, int out_stride, int window) {
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int t = blockIdx.x, h = blockIdx.y, dim = threadIdx.x;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     float* orow = out + (size_t)t * out_stride + (size_t)h * d;
     if (p / FA_CHUNK > nchunks - 1) {
-        for (int dim = lane; dim < d; dim += 64) orow[dim] = __int_as_float(0x7fc00000);
+        if (dim < d) orow[dim] = __int_as_float(0x7fc00000);
         return;
     }
-    float M = -INFINITY, L = 0.f;
-    float ACC[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int c = lo / FA_CHUNK; c <= p / FA_CHUNK; ++c) {
-        const float* src = ws + (((size_t)t * nh + h) * nchunks + c) * (d + FA_WS_PAD);
-        float a, b;
-        fa_fold_scales(M, L, src[d], src[d + 1], a, b);
+    const int dimc = dim < d ? dim : d - 1;
+    const int c_last = p / FA_CHUNK;
+    const float* base = ws + ((size_t)t * nh + h) * nchunks * (d + FA_WS_PAD);
+    float M = -INFINITY, L = 0.f, ACC = 0.f;
+    for (int c0 = lo / FA_CHUNK; c0 <= c_last; c0 += FA_FOLD_AHEAD) {
+        float mm[FA_FOLD_AHEAD], ll[FA_FOLD_AHEAD], av[FA_FOLD_AHEAD];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int dim = lane + 64 * i;
-            if (dim < d) ACC[i] = fmaf(ACC[i], a, src[dim] * b);
+        for (int u = 0; u < FA_FOLD_AHEAD; ++u) {
+            const int c = c0 + u <= c_last ? c0 + u : c_last;
+            const float* src = base + (size_t)c * (d + FA_WS_PAD);
+            mm[u] = src[d];
+            ll[u] = src[d + 1];
+            av[u] = src[dimc];
+        }
+#pragma unroll
+        for (int u = 0; u < FA_FOLD_AHEAD; ++u) {
+            if (c0 + u <= c_last) {
+                float a, b;
+                fa_fold_scales(M, L, mm[u], ll[u], a, b);
+                ACC = fmaf(ACC, a, av[u] * b);
+            }
         }
     }
-    const float inv = 1.0f / L;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int dim = lane + 64 * i;
-        if (dim < d) orow[dim] = ACC[i] * inv;
-    }
+    if (dim < d) orow[dim] = ACC * (1.0f / L);
 }
 
 extern "C" int ilm_attn_f32_chunk() { return FA_CHUNK; }
@@ -279,7 +288,7 @@ extern "C" int ilm_attn_f32(void* out, void* ws, int nchunks, const void* q, con
 #undef FA_ARGS
     ILM_LAUNCH_CHECK("attn_f32");
     if (ws != nullptr) {
-        attn_f32_fold_kernel<<<dim3(T_, nh), 64, 0, stream>>>((float*)out, (const float*)ws, (const int*)pos, nh, d, nchunks,
+        attn_f32_fold_kernel<<<dim3(T_, nh), 64 * ((d + 63) / 64), 0, stream>>>((float*)out, (const float*)ws, (const int*)pos, nh, d, nchunks,
                                                               out_stride, window);
         ILM_LAUNCH_CHECK("attn_f32_fold");
     }

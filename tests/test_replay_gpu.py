@@ -189,3 +189,35 @@ def _mixed_batches_with_page_reuse(case, page):
     assert any(len(h) > 1 for h in holders.values()), "no page was held by two requests: the pool is not small enough"
     assert drv.runner.cache.free_pages() == num_pages
     drv.runner.cache.check()
+    return drv
+
+
+def test_float32_logits_do_not_depend_on_the_cutting_bit_for_bit(case):
+    """In 32-bit every sum has one order, fixed by the operands' shapes and the token's position (products in
+    eight slices of K whatever the number of rows, attention in chunks of 128 keys by absolute index): a request
+    whole, with its last 32 tokens one by one, in portions down to two tokens and mixed with other requests
+    over other page sizes gives the same logits bit for bit, not only within a tolerance."""
+    if case["dtype"] != "float32":
+        pytest.skip("bfloat16 steps of different sizes take different kernels: equal within the tolerance only")
+    runs = {}
+    n0 = len(case["toks"]["r0"])
+    drv = Driver(case["dir"], "float32", num_pages=_pages(n0, 16) + 1, page_size=16)
+    for rid in ("r0", "r3", "r5"):
+        drv.step([(rid, case["toks"][rid])], end=[rid])
+    runs["whole"] = drv
+    drv = Driver(case["dir"], "float32", num_pages=_pages(n0, 8) + 1, page_size=8)
+    _bulk_then_last_32(case, drv)
+    runs["last 32 one by one"] = drv
+    drv = Driver(case["dir"], "float32", num_pages=_pages(n0, 4) + 1, page_size=4)
+    _portions_of_changing_size(case, drv)
+    runs["portions"] = drv
+    runs["mixed"] = _mixed_batches_with_page_reuse(case, 64)
+    for rid in ("r0", "r3", "r5"):
+        n = len(case["toks"][rid])
+        want = runs["whole"].request_logits(rid, n)
+        for name, drv in runs.items():
+            got = drv.request_logits(rid, n)
+            same = torch.equal(got, want)
+            if not same:
+                bad = (got != want).any(dim=1).nonzero()[0].item()
+                assert same, f"{case['name']} request {rid}: '{name}' differs from 'whole' first at position {bad}"
