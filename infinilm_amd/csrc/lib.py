@@ -32,6 +32,15 @@ _SIGNATURES = {
     "ilm_gemm_rows64": [_P, _I, _L, _I, _P, _I, _I, _I, _I, _P, _I, _P],
     "ilm_gemm_mid": [_P, _I, _L, _I, _I, _P, _I, _I, _I, _I, _P, _I, _I, _P],
     "ilm_gemm_qkv_rope": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "ilm_gemm_qkv_rope_wide": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "ilm_gemm_wide": [_P, _I, _L, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _F, _I, _P],
+    "ilm_frag_pack_weight": [_P, _P, _P, _I, _I, _I, _I, _P],
+    "ilm_frag_pack_rows": [_P, _P, _I, _I, _I, _P],
+    "ilm_frag_unpack_rows": [_P, _P, _I, _I, _I, _P],
+    "ilm_gemm_frag": [_P, _I, _L, _I, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P],
+    "ilm_gemm_frag_swiglu": [_P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _F, _I, _P],
+    "ilm_gemm_frag_rope": [_P, _I, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "ilm_gemm_frag_tail": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _P],
     "ilm_gemm_f32_skinny": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
     "ilm_gemm_f32_tile": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
     "ilm_attn_f32": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],

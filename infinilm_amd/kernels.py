@@ -204,6 +204,9 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, 
 
 
 USE_QKV_ROPE = os.environ.get("INFINILM_AMD_QKV_ROPE", "1") == "1"
+# Rows up to which the q/k/v projection with X streamed beside W is used above the few rows (0: never)
+QKV_ROPE_WIDE_ROWS = int(os.environ.get("INFINILM_AMD_QKV_ROPE_WIDE_ROWS", "64"))
+QKV_ROPE_WIDE_PAIRS = int(os.environ.get("INFINILM_AMD_QKV_ROPE_WIDE_PAIRS", "0"))   # pairs a run (0: the kernel chooses)
 
 
 def qkv_rope_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
@@ -211,11 +214,12 @@ def qkv_rope_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
                   slots: Optional[torch.Tensor], nh: int, nkv: int, d: int, rd: int) -> Optional[torch.Tensor]:
     """The fused projection x w^T (+ bias) of a few rows, q and k rotated and k, v written to the cache
     in the product's epilogue.  Returns the rotated q [T, nh*d], or None where the fused kernel does
-    not apply (more than 32 rows, float32, a partly rotated or odd-sized head): the caller then
+    not apply (more than 64 rows, float32, a partly rotated or odd-sized head): the caller then
     runs the projection and `rope_kvwrite` one after the other."""
     M, K = x.shape
-    if not (USE_QKV_ROPE and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and _few_rows(M, K) and rd == d and d % 32 == 0
-            and K % 8 == 0 and K <= 8192 and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
+    wide = not _few_rows(M, K) and 16 < M <= min(QKV_ROPE_WIDE_ROWS, 64)
+    if not (USE_QKV_ROPE and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and (_few_rows(M, K) or wide) and rd == d and d % 32 == 0
+            and K % 8 == 0 and (K <= 8192 or wide) and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
             and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         return None
     _dev(x, w, bias, positions, cos, sin, k_cache, v_cache, slots)
@@ -234,6 +238,11 @@ def qkv_rope_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
             raise KernelError("cache tensors missing or of another dtype than the activations")
         page = _check_cache(k_cache, v_cache, nkv, d)
     q = torch.empty((M, nh * d), dtype=BF16, device=x.device)
+    if wide:
+        _run("ilm_gemm_qkv_rope_wide", q.data_ptr(), q.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
+             _ptr(bias), M, K, positions.data_ptr(), cos.data_ptr(), sin.data_ptr(), _ptr(k_cache) if slots is not None else None,
+             _ptr(v_cache) if slots is not None else None, _ptr(slots), nh, nkv, d, page, QKV_ROPE_WIDE_PAIRS, _stream())
+        return q
     _run("ilm_gemm_qkv_rope", q.data_ptr(), q.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), _ptr(bias),
          M, K, positions.data_ptr(), cos.data_ptr(), sin.data_ptr(), _ptr(k_cache) if slots is not None else None,
          _ptr(v_cache) if slots is not None else None, _ptr(slots), nh, nkv, d, page, _stream())
@@ -675,3 +684,217 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     _run("ilm_sample", out.data_ptr(), logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
          uniform.data_ptr(), n, V, logits.stride(0), _stream())
     return out
+
+
+# ---- operands in fragment order (csrc/frag.h): the products of a decode step ------------------------------
+FRAG_MAX_ROWS = 64    # most rows of X the fragment-order products take
+FRAG_SS_ROWS = 64     # rows of a tile's record of partial sums of squares (ilm_gemm_frag_ss_rows())
+USE_FRAG = os.environ.get("INFINILM_AMD_FRAG", "1") == "1" and not FORCE_BASIC
+FRAG_TILES = int(os.environ.get("INFINILM_AMD_FRAG_TILES", "2"))   # tiles of W a workgroup (2 or 4)
+
+
+class FragRows:
+    """Activations [rows, width] in bfloat16, stored in fragment order (`data`: a flat int32 buffer)."""
+    __slots__ = ("data", "rows", "width")
+
+    def __init__(self, data: torch.Tensor, rows: int, width: int):
+        self.data, self.rows, self.width = data, int(rows), int(width)
+
+    @property
+    def shape(self):
+        return (self.rows, self.width)
+
+    @property
+    def dtype(self):
+        return BF16
+
+    @property
+    def device(self):
+        return self.data.device
+
+
+def frag_rows_empty(rows: int, width: int, device) -> FragRows:
+    """An uninitialised fragment-order buffer for [rows, width]; the k beyond the width (up to a multiple of 32)
+    are zeros, as the products need them."""
+    groups, steps = -(-rows // 16), -(-width // 32)
+    if width % 32:
+        data = torch.zeros((steps * groups * 64 * 4,), dtype=torch.int32, device=device)
+    else:
+        data = torch.empty((steps * groups * 64 * 4,), dtype=torch.int32, device=device)
+    return FragRows(data, rows, width)
+
+
+def to_frag(x: torch.Tensor) -> FragRows:
+    """Plain bfloat16 rows into fragment order (a kernel of its own: for producers that have no such store)."""
+    _dev(x)
+    M, K = x.shape
+    if x.dtype != BF16 or x.stride(1) != 1 or K % 8 or x.stride(0) % 8 or x.data_ptr() % 16:
+        raise KernelError("fragment order takes bfloat16 rows of a multiple of 8 elements, 16-byte aligned")
+    out = FragRows(torch.empty((-(-K // 32) * -(-M // 16) * 64 * 4,), dtype=torch.int32, device=x.device), M, K)
+    _run("ilm_frag_pack_rows", out.data.data_ptr(), x.data_ptr(), M, K, x.stride(0), _stream())
+    return out
+
+
+def from_frag(f: FragRows) -> torch.Tensor:
+    out = torch.empty((f.rows, f.width), dtype=BF16, device=f.data.device)
+    _run("ilm_frag_unpack_rows", out.data_ptr(), f.data.data_ptr(), f.rows, f.width, f.width, _stream())
+    return out
+
+
+class FragWeight:
+    """A weight [N, K] in fragment order: tiles of 16 rows in the order `rows` names (None: W's own), padded to a
+    multiple of 4 tiles; `tiles` counts the real ones."""
+    __slots__ = ("data", "N", "K", "tiles", "kind")
+
+    def __init__(self, data, N, K, tiles, kind):
+        self.data, self.N, self.K, self.tiles, self.kind = data, N, K, tiles, kind
+
+
+def frag_weight_ok(w: torch.Tensor) -> bool:
+    return (USE_FRAG and w.is_cuda and w.dtype == BF16 and w.dim() == 2 and w.shape[1] % 8 == 0 and w.stride(1) == 1
+            and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0)
+
+
+def pack_weight(w: torch.Tensor, kind: str = "plain", **layout) -> FragWeight:
+    """`kind`: "plain" (tiles of consecutive rows), "gate_up" (w = [Wg; Wu]: tile pairs (gate rows 16p.., up rows 16p..)),
+    "qkv" (nh, nkv, d given: tile pairs (first rows, second rows) of 16 rotation pairs; pair p = head slot p // (d/2),
+    dim p % (d/2))."""
+    if not frag_weight_ok(w):
+        raise KernelError("fragment order takes a bfloat16 weight with rows of a multiple of 8 elements, 16-byte aligned")
+    N, K = w.shape
+    rows = None
+    if kind == "plain":
+        tiles = -(-N // 16)
+    elif kind == "gate_up":
+        I = N // 2
+        it = -(-I // 16)
+        idx = torch.arange(it * 16, dtype=torch.int64).view(it, 16)
+        g = torch.where(idx < I, idx, torch.full_like(idx, -1))
+        u = torch.where(idx < I, idx + I, torch.full_like(idx, -1))
+        rows = torch.stack([g, u], dim=1).reshape(-1)
+        tiles = 2 * it
+    elif kind == "qkv":
+        nh, nkv, d = layout["nh"], layout["nkv"], layout["d"]
+        half = d // 2
+        pairs = (nh + 2 * nkv) * half
+        pt = -(-pairs // 16)
+        p = torch.arange(pt * 16, dtype=torch.int64).view(pt, 16)
+        first = (p // half) * d + p % half
+        a = torch.where(p < pairs, first, torch.full_like(p, -1))
+        b = torch.where(p < pairs, first + half, torch.full_like(p, -1))
+        rows = torch.stack([a, b], dim=1).reshape(-1)
+        tiles = 2 * pt
+    else:
+        raise KernelError(f"unknown fragment layout {kind!r}")
+    alloc = -(-tiles // 4) * 4
+    steps = -(-K // 32)
+    data = torch.zeros((alloc * steps * 64 * 4,), dtype=torch.int32, device=w.device)
+    rows_dev = None
+    if rows is not None:
+        rows_dev = rows.to(torch.int32).to(w.device)
+    _run("ilm_frag_pack_weight", data.data_ptr(), w.data_ptr(), _ptr(rows_dev), N, K, w.stride(0), tiles, _stream())
+    return FragWeight(data, N, K, tiles, kind)
+
+
+def _frag_x(x: FragRows, fw: FragWeight) -> None:
+    if not isinstance(x, FragRows) or x.width != fw.K or x.rows > FRAG_MAX_ROWS:
+        raise KernelError(f"fragment-order product: X {getattr(x, 'shape', None)} does not fit W [{fw.N}, {fw.K}] "
+                          f"(at most {FRAG_MAX_ROWS} rows)")
+
+
+def gemm_frag(x: FragRows, fw: FragWeight, bias: Optional[torch.Tensor] = None, alpha: float = 1.0,
+              out: str = "bf16", parts: int = 1):
+    """alpha (x W^T + bias) of up to 64 rows.  `out`: "bf16" or "f32" rows [M, N]; "parts": float32 [parts, M, N] of a
+    K split in `parts` ranges (for add_rmsnorm); "frag": bfloat16 in fragment order."""
+    _frag_x(x, fw)
+    M, N, K = x.rows, fw.N, fw.K
+    steps = -(-K // 32)
+    spp = 0
+    if out == "parts":
+        spp = -(-steps // max(parts, 1))
+        spp = -(-spp // 8) * 8 if spp > 8 else spp
+        parts = -(-steps // spp)
+        res = torch.empty((parts, M, N), dtype=F32, device=x.device)
+        kind, ldc, target = 1, N, res
+    elif out == "f32":
+        res = torch.empty((M, N), dtype=F32, device=x.device)
+        kind, ldc, target = 1, N, res
+    elif out == "bf16":
+        res = torch.empty((M, N), dtype=BF16, device=x.device)
+        kind, ldc, target = 0, N, res
+    else:
+        res = frag_rows_empty(M, N, x.device)
+        kind, ldc, target = 2, N, res.data
+    if bias is not None and (bias.shape != (N,) or bias.dtype != BF16 or not bias.is_contiguous()):
+        raise KernelError("bias does not fit the product")
+    _run("ilm_gemm_frag", target.data_ptr(), ldc, M * N, kind, x.data.data_ptr(), fw.data.data_ptr(), _ptr(bias), M, N, K,
+         spp, float(alpha), FRAG_TILES, _stream())
+    return res
+
+
+def gemm_frag_swiglu(x: FragRows, fw: FragWeight, bias: Optional[torch.Tensor] = None,
+                     row_ss: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0) -> FragRows:
+    """silu(x Wg^T + bg) * (x Wu^T + bu) in fragment order; `row_ss`: x is what `gemm_frag_tail` left and the rows'
+    division by sqrt(mean square + eps) over `norm_width` happens here."""
+    _frag_x(x, fw)
+    if fw.kind != "gate_up":
+        raise KernelError("the SwiGLU epilogue needs a weight packed as gate_up")
+    I = fw.N // 2
+    if bias is not None and (bias.shape != (2 * I,) or bias.dtype != BF16 or not bias.is_contiguous()):
+        raise KernelError("bias does not fit the fused gate/up projection")
+    if row_ss is not None and (row_ss.dtype != F32 or row_ss.dim() != 2 or row_ss.shape[1] != FRAG_SS_ROWS or not row_ss.is_contiguous()):
+        raise KernelError("partial sums of squares must be float32 [tiles, 64]")
+    act = frag_rows_empty(x.rows, I, x.device)
+    _run("ilm_gemm_frag_swiglu", act.data.data_ptr(), x.data.data_ptr(), fw.data.data_ptr(), _ptr(bias), x.rows, I, fw.K,
+         _ptr(row_ss), 0 if row_ss is None else row_ss.shape[0], int(norm_width), float(eps), FRAG_TILES, _stream())
+    return act
+
+
+def gemm_frag_rope(x: FragRows, fw: FragWeight, bias: Optional[torch.Tensor], positions: torch.Tensor, cos: torch.Tensor,
+                   sin: torch.Tensor, k_cache, v_cache, slots, nh: int, nkv: int, d: int) -> torch.Tensor:
+    """The fused q/k/v projection with rotation and cache write; returns the rotated q [M, nh*d]."""
+    _frag_x(x, fw)
+    if fw.kind != "qkv" or fw.N != (nh + 2 * nkv) * d or d % 32:
+        raise KernelError("the rotation epilogue needs a weight packed as qkv with heads in steps of 32")
+    M = x.rows
+    _i32(positions, "positions")
+    if positions.numel() != M:
+        raise KernelError("positions must have one entry a row")
+    if cos.dtype != F32 or sin.dtype != F32 or cos.shape != sin.shape or cos.shape[1] != d // 2 \
+            or not cos.is_contiguous() or not sin.is_contiguous():
+        raise KernelError(f"rotation tables must be float32 [positions, {d // 2}], got {tuple(cos.shape)}")
+    if bias is not None and (bias.shape != (fw.N,) or bias.dtype != BF16 or not bias.is_contiguous()):
+        raise KernelError("bias does not fit the fused projection")
+    page = 0
+    if slots is not None:
+        _i32(slots, "slots")
+        if k_cache is None or v_cache is None or k_cache.dtype != BF16 or v_cache.dtype != BF16:
+            raise KernelError("cache tensors missing or of another dtype than the activations")
+        page = _check_cache(k_cache, v_cache, nkv, d)
+    q = torch.empty((M, nh * d), dtype=BF16, device=x.device)
+    _run("ilm_gemm_frag_rope", q.data_ptr(), q.stride(0), x.data.data_ptr(), fw.data.data_ptr(), _ptr(bias), M, fw.K,
+         positions.data_ptr(), cos.data_ptr(), sin.data_ptr(), _ptr(k_cache) if slots is not None else None,
+         _ptr(v_cache) if slots is not None else None, _ptr(slots), nh, nkv, d, page, _stream())
+    return q
+
+
+def gemm_frag_tail(x: FragRows, fw: FragWeight, bias: Optional[torch.Tensor], alpha: float, residual: torch.Tensor,
+                   norm_w: torch.Tensor):
+    """residual += alpha (x W^T + bias) in place; returns (xw, ss): xw = bfloat16(residual * norm_w) in fragment order,
+    ss [ceil(N / 16), 64] partial sums of squares of the residual's rows."""
+    _frag_x(x, fw)
+    M, N = x.rows, fw.N
+    if fw.kind != "plain":
+        raise KernelError("the tail epilogue needs a weight packed plainly")
+    if residual.dtype != F32 or tuple(residual.shape) != (M, N) or residual.stride(1) != 1:
+        raise KernelError("the residual stream is a float32 tensor with dense rows of the product's width")
+    if norm_w.shape != (N,) or norm_w.dtype not in (BF16, F32) or not norm_w.is_contiguous():
+        raise KernelError("the norm's weight does not fit")
+    if bias is not None and (bias.shape != (N,) or bias.dtype != BF16 or not bias.is_contiguous()):
+        raise KernelError("bias does not fit the product")
+    xw = frag_rows_empty(M, N, x.device)
+    ss = torch.empty((-(-N // 16), FRAG_SS_ROWS), dtype=F32, device=x.device)
+    _run("ilm_gemm_frag_tail", residual.data_ptr(), residual.stride(0), xw.data.data_ptr(), ss.data_ptr(), x.data.data_ptr(),
+         fw.data.data_ptr(), _ptr(bias), norm_w.data_ptr(), 1 if norm_w.dtype == F32 else 0, float(alpha), M, N, fw.K,
+         FRAG_TILES, _stream())
+    return xw, ss
