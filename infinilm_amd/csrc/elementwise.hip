@@ -3,6 +3,7 @@
 #include <stdarg.h>
 
 #include "common.h"
+#include "frag.h"
 
 static thread_local char g_err[1024] = {0};
 
@@ -73,7 +74,7 @@ __device__ __forceinline__ void load8(const T* p, float* v) {
 template <typename T, typename WT, typename HT>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __restrict__ h,
-                   const WT* __restrict__ w, int H, float alpha, float eps, int parts, size_t pstride) {
+                   const WT* __restrict__ w, int H, float alpha, float eps, int parts, size_t pstride, int frag_mg) {
     __shared__ float red[4];
     const size_t base = (size_t)blockIdx.x * H;
     float ss = 0.f;
@@ -93,6 +94,13 @@ add_rmsnorm_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __restric
     }
     const float tot = block_sum<4>(ss, red);
     const float rstd = 1.0f / sqrtf(tot / (float)H + eps);
+    if (frag_mg > 0) {
+        // fragment order (frag.h), H a multiple of 8; the k up to the next multiple of 32 are zeros
+        const int kp = (H + 31) / 32 * 32;
+        for (int j = threadIdx.x; j < kp; j += 256)
+            x[frag_x_chunk(blockIdx.x, j >> 3, frag_mg) * 8 + (j & 7)] = from_f32<T>(j < H ? r[base + j] * rstd * to_f32(w[j]) : 0.f);
+        return;
+    }
     for (int j = threadIdx.x; j < H; j += 256)
         x[base + j] = from_f32<T>(r[base + j] * rstd * to_f32(w[j]));
 }
@@ -103,7 +111,7 @@ add_rmsnorm_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __restric
 template <typename T, typename WT, typename HT, int NITER>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __restrict__ h,
-                       const WT* __restrict__ w, int H, float alpha, float eps, int parts, size_t pstride) {
+                       const WT* __restrict__ w, int H, float alpha, float eps, int parts, size_t pstride, int frag_mg) {
     __shared__ float red[4];
     const size_t base = (size_t)blockIdx.x * H;
     float v[NITER][8];
@@ -166,7 +174,9 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __res
             T o[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) o[e] = from_f32<T>(v[it][e] * rstd * wv[it][e]);
-            if (sizeof(T) == 2) {
+            if (sizeof(T) == 2 && frag_mg > 0) {   // fragment order (frag.h): the 16-byte chunk of row blockIdx.x
+                reinterpret_cast<uint4*>(x)[frag_x_chunk(blockIdx.x, j >> 3, frag_mg)] = *reinterpret_cast<uint4*>(o);
+            } else if (sizeof(T) == 2) {
                 *reinterpret_cast<uint4*>(x + base + j) = *reinterpret_cast<uint4*>(o);
             } else {
                 *reinterpret_cast<float4*>(x + base + j) = *reinterpret_cast<float4*>(o);
@@ -174,14 +184,21 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __res
             }
         }
     }
+    if (sizeof(T) == 2 && frag_mg > 0) {   // the k up to the next multiple of 32 are zeros
+        for (int k8 = (H >> 3) + threadIdx.x; k8 < (H + 31) / 32 * 4; k8 += 256)
+            reinterpret_cast<uint4*>(x)[frag_x_chunk(blockIdx.x, k8, frag_mg)] = make_uint4(0u, 0u, 0u, 0u);
+    }
 }
 
 // h: the pending branch [parts][rows][H] in the activations' dtype (h_dtype == dtype) or in float
 // (h_dtype == ILM_DTYPE_F32, e.g. the parts of a K-split product); null: nothing to add.
 extern "C" int ilm_add_rmsnorm(void* x, void* r, const void* h, const void* w, int rows, int H,
                                float alpha, float eps, int dtype, int w_dtype, int h_dtype, int parts,
-                               long pstride, hipStream_t stream) {
+                               long pstride, int frag_mg, hipStream_t stream) {
+    // frag_mg > 0: x is bfloat16 in fragment order (frag.h) with frag_mg = ceil(rows / 16) groups of rows
     ILM_REQUIRE(rows > 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", rows, H);
+    ILM_REQUIRE(frag_mg == 0 || (dtype == ILM_DTYPE_BF16 && H % 8 == 0 && frag_mg == (rows + 15) / 16),
+                "add_rmsnorm: a result in fragment order is bfloat16 with rows of a multiple of 8 elements");
     ILM_REQUIRE(h == nullptr || (parts >= 1 && (h_dtype == dtype || h_dtype == ILM_DTYPE_F32)),
                 "add_rmsnorm: the branch must have the activations' dtype or be float, in >= 1 parts");
     // H a multiple of 8 up to 8192 with 16-byte aligned rows takes the vector kernel
@@ -192,13 +209,13 @@ extern "C" int ilm_add_rmsnorm(void* x, void* r, const void* h, const void* w, i
 #define NORM_LAUNCH(T, WT, HT)                                                                                   \
     do {                                                                                                         \
         if (vec && niter <= 1)                                                                                   \
-            add_rmsnorm_vec_kernel<T, WT, HT, 1><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride); \
+            add_rmsnorm_vec_kernel<T, WT, HT, 1><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride, frag_mg); \
         else if (vec && niter <= 2)                                                                              \
-            add_rmsnorm_vec_kernel<T, WT, HT, 2><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride); \
+            add_rmsnorm_vec_kernel<T, WT, HT, 2><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride, frag_mg); \
         else if (vec)                                                                                            \
-            add_rmsnorm_vec_kernel<T, WT, HT, 4><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride); \
+            add_rmsnorm_vec_kernel<T, WT, HT, 4><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride, frag_mg); \
         else                                                                                                     \
-            add_rmsnorm_kernel<T, WT, HT><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride); \
+            add_rmsnorm_kernel<T, WT, HT><<<rows, 256, 0, stream>>>((T*)x, (float*)r, (const HT*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride, frag_mg); \
     } while (0)
 #define NORM_CASE(T, WT)                     \
     do {                                     \

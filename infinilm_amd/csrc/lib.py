@@ -20,7 +20,7 @@ _L = c_long
 
 _SIGNATURES = {
     "ilm_embed": [_P, _P, _P, _I, _I, _I, _F, _I, _P],
-    "ilm_add_rmsnorm": [_P, _P, _P, _P, _I, _I, _F, _F, _I, _I, _I, _I, _L, _P],
+    "ilm_add_rmsnorm": [_P, _P, _P, _P, _I, _I, _F, _F, _I, _I, _I, _I, _L, _I, _P],
     "ilm_gemm_ksplit": [_P, _I, _I, _L, _I, _P, _I, _P, _F, _I, _I, _I, _P, _I, _I, _P],
     "ilm_rope_kvwrite": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "ilm_swiglu": [_P, _P, _I, _I, _I, _I, _P],
@@ -32,8 +32,6 @@ _SIGNATURES = {
     "ilm_gemm_rows64": [_P, _I, _L, _I, _P, _I, _I, _I, _I, _P, _I, _P],
     "ilm_gemm_mid": [_P, _I, _L, _I, _I, _P, _I, _I, _I, _I, _P, _I, _I, _P],
     "ilm_gemm_qkv_rope": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
-    "ilm_gemm_qkv_rope_wide": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
-    "ilm_gemm_wide": [_P, _I, _L, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _F, _I, _P],
     "ilm_frag_pack_weight": [_P, _P, _P, _I, _I, _I, _I, _P],
     "ilm_frag_pack_rows": [_P, _P, _I, _I, _I, _P],
     "ilm_frag_unpack_rows": [_P, _P, _I, _I, _I, _P],

@@ -156,8 +156,10 @@ def embed(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
 
 
 def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: torch.Tensor,
-                alpha: float, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+                alpha: float, eps: float, out_dtype: torch.dtype, frag: bool = False):
     """residual += alpha * branch (in place, float32), then its RMS norm times weight, as out_dtype.
+    `frag`: the result comes in fragment order (`FragRows`; bfloat16, at most 64 rows of a multiple of 8 elements),
+    for a product that takes it so.
 
     `branch` is [rows, H] in out_dtype or float32, or [parts, rows, H] (the float32 parts of a K-split
     product, summed in order)."""
@@ -175,9 +177,16 @@ def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: 
         h_dt = _dt(branch)
     if weight.shape != (H,) or not weight.is_contiguous():
         raise KernelError(f"norm weight has shape {tuple(weight.shape)}, expected ({H},)")
+    if frag:
+        if out_dtype != BF16 or rows > FRAG_MAX_ROWS or H % 8:
+            raise KernelError("a norm's result in fragment order is bfloat16, at most 64 rows of a multiple of 8 elements")
+        out = frag_rows_empty(rows, H, residual.device)
+        _run("ilm_add_rmsnorm", out.data.data_ptr(), residual.data_ptr(), _ptr(branch), weight.data_ptr(), rows, H,
+             float(alpha), float(eps), _DT[out_dtype], _dt(weight), h_dt, parts, pstride, -(-rows // 16), _stream())
+        return out
     out = torch.empty((rows, H), dtype=out_dtype, device=residual.device)
     _run("ilm_add_rmsnorm", out.data_ptr(), residual.data_ptr(), _ptr(branch), weight.data_ptr(), rows, H,
-         float(alpha), float(eps), _DT[out_dtype], _dt(weight), h_dt, parts, pstride, _stream())
+         float(alpha), float(eps), _DT[out_dtype], _dt(weight), h_dt, parts, pstride, 0, _stream())
     return out
 
 
@@ -204,9 +213,6 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, 
 
 
 USE_QKV_ROPE = os.environ.get("INFINILM_AMD_QKV_ROPE", "1") == "1"
-# Rows up to which the q/k/v projection with X streamed beside W is used above the few rows (0: never)
-QKV_ROPE_WIDE_ROWS = int(os.environ.get("INFINILM_AMD_QKV_ROPE_WIDE_ROWS", "64"))
-QKV_ROPE_WIDE_PAIRS = int(os.environ.get("INFINILM_AMD_QKV_ROPE_WIDE_PAIRS", "0"))   # pairs a run (0: the kernel chooses)
 
 
 def qkv_rope_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
@@ -214,12 +220,11 @@ def qkv_rope_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
                   slots: Optional[torch.Tensor], nh: int, nkv: int, d: int, rd: int) -> Optional[torch.Tensor]:
     """The fused projection x w^T (+ bias) of a few rows, q and k rotated and k, v written to the cache
     in the product's epilogue.  Returns the rotated q [T, nh*d], or None where the fused kernel does
-    not apply (more than 64 rows, float32, a partly rotated or odd-sized head): the caller then
+    not apply (more than 32 rows, float32, a partly rotated or odd-sized head): the caller then
     runs the projection and `rope_kvwrite` one after the other."""
     M, K = x.shape
-    wide = not _few_rows(M, K) and 16 < M <= min(QKV_ROPE_WIDE_ROWS, 64)
-    if not (USE_QKV_ROPE and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and (_few_rows(M, K) or wide) and rd == d and d % 32 == 0
-            and K % 8 == 0 and (K <= 8192 or wide) and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
+    if not (USE_QKV_ROPE and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and _few_rows(M, K) and rd == d and d % 32 == 0
+            and K % 8 == 0 and K <= 8192 and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
             and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         return None
     _dev(x, w, bias, positions, cos, sin, k_cache, v_cache, slots)
@@ -238,11 +243,6 @@ def qkv_rope_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
             raise KernelError("cache tensors missing or of another dtype than the activations")
         page = _check_cache(k_cache, v_cache, nkv, d)
     q = torch.empty((M, nh * d), dtype=BF16, device=x.device)
-    if wide:
-        _run("ilm_gemm_qkv_rope_wide", q.data_ptr(), q.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
-             _ptr(bias), M, K, positions.data_ptr(), cos.data_ptr(), sin.data_ptr(), _ptr(k_cache) if slots is not None else None,
-             _ptr(v_cache) if slots is not None else None, _ptr(slots), nh, nkv, d, page, QKV_ROPE_WIDE_PAIRS, _stream())
-        return q
     _run("ilm_gemm_qkv_rope", q.data_ptr(), q.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), _ptr(bias),
          M, K, positions.data_ptr(), cos.data_ptr(), sin.data_ptr(), _ptr(k_cache) if slots is not None else None,
          _ptr(v_cache) if slots is not None else None, _ptr(slots), nh, nkv, d, page, _stream())
@@ -794,6 +794,18 @@ def pack_weight(w: torch.Tensor, kind: str = "plain", **layout) -> FragWeight:
         rows_dev = rows.to(torch.int32).to(w.device)
     _run("ilm_frag_pack_weight", data.data_ptr(), w.data_ptr(), _ptr(rows_dev), N, K, w.stride(0), tiles, _stream())
     return FragWeight(data, N, K, tiles, kind)
+
+
+# Rows from which the q/k/v projection of a decode step takes its operands in fragment order (measured at the 8B
+# shape: 12.7 against 17.3 us at 32 rows, 16.2 against 22.5 us for the vendor library's product and the rotation
+# kernel at 64; up to 16 rows the kernel that keeps X in registers is as fast)
+FRAG_QKV_MIN_ROWS = int(os.environ.get("INFINILM_AMD_FRAG_QKV_MIN_ROWS", "17"))
+
+
+def qkv_frag_ok(rows: int, w: torch.Tensor, d: int, rd: int, width: int) -> bool:
+    """Whether the fused q/k/v projection takes `rows` rows in fragment order (see `gemm_frag_rope`)."""
+    return (FRAG_QKV_MIN_ROWS <= rows <= FRAG_MAX_ROWS and frag_weight_ok(w) and rd == d and d % 32 == 0 and width % 8 == 0
+            and USE_QKV_ROPE)
 
 
 def _frag_x(x: FragRows, fw: FragWeight) -> None:

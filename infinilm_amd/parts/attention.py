@@ -48,7 +48,11 @@ class GQAttention(Mixer):
 
     takes_tail = True
 
-    def forward(self, x: torch.Tensor, batch, cache_view, tail=None):
+    def takes_frag(self, rows: int) -> bool:
+        fn = getattr(self.position, "takes_frag", None)
+        return bool(fn is not None and fn(rows, self.qkv, self.nh, self.nkv, self.d))
+
+    def forward(self, x, batch, cache_view, tail=None):
         pe = self.position
         pe.check(batch)
         qkv = None

@@ -92,6 +92,10 @@ class DeferredNorm:
 
 
 class Norm(Part):
+    """`takes_frag_request`: forward accepts `frag=True` and then returns its rows in fragment order
+    (`kernels.FragRows`) for a consumer that said `takes_frag(rows)`."""
+    takes_frag_request = False
+
     def forward(self, stream: ResidualStream) -> torch.Tensor:
         raise NotImplementedError
 
@@ -103,6 +107,10 @@ class Norm(Part):
 class Mixer(Part):
     """`takes_tail`: forward accepts `tail=NormTail` and may answer with a DeferredNorm."""
     takes_tail = False
+
+    def takes_frag(self, rows: int) -> bool:
+        """Whether forward accepts x as `kernels.FragRows` (rows in fragment order) for a step of `rows` rows."""
+        return False
 
     def cache_need(self):
         return None

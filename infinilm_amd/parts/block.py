@@ -37,7 +37,13 @@ class PreNormBlock:
         return self.mixer.cache_need()
 
     def forward(self, stream: ResidualStream, batch, cache_view) -> None:
-        x = self.norm1.forward(stream)
+        # a decode step of many rows: the mixer may take its rows in fragment order, which the norm then writes
+        rows = stream.residual.shape[0]
+        if (batch.taps is None and getattr(self.norm1, "takes_frag_request", False)
+                and getattr(self.mixer, "takes_frag", lambda rows: False)(rows)):
+            x = self.norm1.forward(stream, frag=True)
+        else:
+            x = self.norm1.forward(stream)
         # Few rows (decoded tokens): where the mixer's last projection, the second norm and the feed-forward
         # all can, the projection adds into the residual stream itself and the norm's kernel is not run
         # (see NormTail).  Not while intermediate values are dumped: they are taken between the kernels.

@@ -26,6 +26,7 @@ class FusedLinear:
         n = sum(self.out_sizes)
         self.weight = torch.empty((n, self.in_features), dtype=ctx.dtype, device=ctx.device)
         self.bias = torch.empty((n,), dtype=ctx.dtype, device=ctx.device) if bias else None
+        self._frag = {}   # layout -> (version of the weight it was packed from, the weight in fragment order)
 
     def named_parameters(self) -> Dict[str, Param]:
         out: Dict[str, Param] = {}
@@ -36,6 +37,16 @@ class FusedLinear:
                 out[f"{name}.bias"] = Param(self.bias[row:row + size])
             row += size
         return out
+
+    def frag_weight(self, kind: str = "plain", **layout):
+        """The weight in fragment order (`kernels.pack_weight`), packed at its first use and again when the weight
+        has been written since (a second copy of the weight: the many-rows products keep the plain rows)."""
+        key = (kind, tuple(sorted(layout.items())))
+        held = self._frag.get(key)
+        if held is None or held[0] != self.weight._version or held[2] != self.weight.data_ptr():
+            held = (self.weight._version, kernels.pack_weight(self.weight, kind, **layout), self.weight.data_ptr())
+            self._frag[key] = held
+        return held[1]
 
     def forward(self, x: torch.Tensor, alpha: float = 1.0, out_dtype: Optional[torch.dtype] = None,
                 allow_parts: bool = False) -> torch.Tensor:

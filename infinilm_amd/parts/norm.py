@@ -18,6 +18,8 @@ from .registry import register_norm
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
+    takes_frag_request = True
+
     def __init__(self, size: int, eps: float, ctx: BuildContext):
         self.size = int(size)
         self.eps = float(eps)
@@ -35,9 +37,10 @@ class RMSNorm(Norm):
             return None
         return NormTail(stream.residual, float(scale), self.weight, self.eps)
 
-    def forward(self, stream: ResidualStream) -> torch.Tensor:
+    def forward(self, stream: ResidualStream, frag: bool = False):
+        """`frag`: the consumer takes its rows in fragment order (`kernels.FragRows`)."""
         x = kernels.add_rmsnorm(stream.residual, stream.pending, self.weight, stream.pending_scale, self.eps,
-                                self.dtype)
+                                self.dtype, frag=frag)
         stream.pending = None
         stream.pending_scale = 1.0
         return x

@@ -143,8 +143,14 @@ class RotaryEmbedding(PositionEncoding):
         ang = p[:, None] * inv_freq[None, :]
         return (torch.cos(ang) * m).to(torch.float32).contiguous(), (torch.sin(ang) * m).to(torch.float32).contiguous()
 
+    def takes_frag(self, rows, proj, nh, nkv, d):
+        return kernels.qkv_frag_ok(rows, proj.weight, d, self.rotary_dim, proj.in_features)
+
     def project_encode_store(self, x, proj, batch, view, nh, nkv, d):
         # few rows (decoded tokens): projection, rotation and cache write are one kernel
+        if isinstance(x, kernels.FragRows):   # rows in fragment order, as `takes_frag` offered
+            return kernels.gemm_frag_rope(x, proj.frag_weight("qkv", nh=nh, nkv=nkv, d=d), proj.bias, batch.positions,
+                                          self.cos, self.sin, view.k, view.v, view.slots, nh, nkv, d)
         return kernels.qkv_rope_gemm(x, proj.weight, proj.bias, batch.positions, self.cos, self.sin, view.k, view.v,
                                      view.slots, nh, nkv, d, self.rotary_dim)
 
@@ -161,6 +167,9 @@ class NoPositionEncoding(RotaryEmbedding):
         self.head_dim, self.rotary_dim, self.max_positions = int(head_dim), 0, 1 << 30
         self.cos = torch.zeros((1, 0), dtype=torch.float32, device=ctx.device)
         self.sin = torch.zeros((1, 0), dtype=torch.float32, device=ctx.device)
+
+    def takes_frag(self, rows, proj, nh, nkv, d):
+        return False
 
     def project_encode_store(self, x, proj, batch, view, nh, nkv, d):
         return None
