@@ -66,6 +66,9 @@ class ModelSpec:
     # the embedding: a part of kind `embed_kind` built from (vocab_size, hidden_size, scale=embed_scale, **embed_params)
     embed_kind: str = "scaled_lookup"
     embed_params: Dict[str, Any] = field(default_factory=dict)
+    # axes of the positions a step carries for every token (1: the place in the sequence alone; a position encoding
+    # over several axes, rows and columns of a picture beside the place in the text, reads `batch.position_axes`)
+    position_axes: int = 1
 
     def num_cache_entries(self) -> int:
         ids = [r.cache for r in self.order if r.cache is not None]

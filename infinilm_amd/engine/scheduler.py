@@ -81,15 +81,15 @@ class Scheduler:
         if n >= self.max_positions:
             self._fail(req, f"prompt of {n} tokens leaves no room under max_position_embeddings {self.max_positions}")
             return
-        smallest_pool = min((g.pool.num_pages for g in self.cache.groups), default=1 << 30)
-        if self._pages_for(n + 1) > smallest_pool:
-            self._fail(req, f"no_capacity: prompt of {n} tokens needs {self._pages_for(n + 1)} pages, the pool has {smallest_pool}")
-            return
-        if self.policy == "reserve_full":
-            worst = self._pages_for(min(n + req.sampling_params.max_tokens, self.max_positions))
-            if worst > smallest_pool:
-                self._fail(req, f"no_capacity: prompt and max_tokens need {worst} pages, the pool has {smallest_pool}")
+        for g in self.cache.groups:
+            if self._group_pages(g, n + 1) > g.pool.num_pages:
+                self._fail(req, f"no_capacity: prompt of {n} tokens needs {self._group_pages(g, n + 1)} pages, the pool has {g.pool.num_pages}")
                 return
+            if self.policy == "reserve_full":
+                worst = self._group_pages(g, min(n + req.sampling_params.max_tokens, self.max_positions))
+                if worst > g.pool.num_pages:
+                    self._fail(req, f"no_capacity: prompt and max_tokens need {worst} pages, the pool has {g.pool.num_pages}")
+                    return
         req.status = RequestStatus.WAITING
         self.waiting.append(req)
 
@@ -111,11 +111,23 @@ class Scheduler:
         for i, k in enumerate(self.cache.pages_needed(req.request_id, n)):
             promised[i] += k
 
-    def _worst_case_pages(self, req: InferenceRequest) -> int:
-        """Pages the request may still take: up to prompt + max_tokens (scheduler.py:453-495)."""
+    def _group_pages(self, group, n_tokens: int) -> int:
+        """Pages of `group` that a request of `n_tokens` tokens holds at most at any time.  A group that keeps a
+        window gives pages back as the window passes them: a request never holds more than the window, the
+        longest portion of a step, and the page in which the window's edge lies."""
+        pages = self._pages_for(n_tokens)
+        if group.window > 0:
+            pages = min(pages, self._pages_for(group.window + min(self.chunk_size, self.max_num_batched_tokens)) + 1)
+        return pages
+
+    def _worst_case_pages(self, req: InferenceRequest) -> List[int]:
+        """Pages of each group the request may still take: up to prompt + max_tokens (scheduler.py:453-495)."""
         total = min(req.get_prompt_length() + req.sampling_params.max_tokens, self.max_positions)
-        held = len(self.cache.table(req.request_id, 0)) if self.cache.has(req.request_id) and self.cache.groups else 0
-        return max(0, self._pages_for(total) - held)
+        out = []
+        for gi, g in enumerate(self.cache.groups):
+            held = sum(1 for p in self.cache.table(req.request_id, gi) if p >= 0) if self.cache.has(req.request_id) else 0
+            out.append(max(0, self._group_pages(g, total) - held))
+        return out
 
     def _can_admit(self, req: InferenceRequest, first_portion_end: int, promised: List[int],
                    shared_pages: int = 0, shared_idle: int = 0) -> bool:
@@ -123,9 +135,14 @@ class Scheduler:
         takes over from published pages; `shared_idle` of those are idle now, so taking them over
         leaves that many fewer pages to give out."""
         if self.policy == "reserve_full":
-            need = self._pages_for(min(req.get_prompt_length() + req.sampling_params.max_tokens, self.max_positions))
-            need += sum(self._worst_case_pages(r) for r in self.running) - shared_pages + shared_idle
-            return all(need <= g.pool.num_free for g in self.cache.groups)
+            # every group by its own need (scheduler.py:453-495 has one pool; here the groups differ: all keys, a window)
+            total = min(req.get_prompt_length() + req.sampling_params.max_tokens, self.max_positions)
+            running = [self._worst_case_pages(r) for r in self.running]
+            for gi, g in enumerate(self.cache.groups):
+                need = self._group_pages(g, total) + sum(w[gi] for w in running) - shared_pages + shared_idle
+                if need > g.pool.num_free:
+                    return False
+            return True
         need = self._pages_for(first_portion_end) - shared_pages + shared_idle
         return all(p + need <= g.pool.num_free for p, g in zip(promised, self.cache.groups))
 

@@ -27,6 +27,9 @@ class StepEntry:
     req_id: object
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    # for models whose positions have several axes (`ModelSpec.position_axes`): [axes][len(tokens)] positions for
+    # the encoding; None: every axis is the token's place in its sequence
+    positions: Optional[Sequence[Sequence[int]]] = None
 
 
 class StepBatch:
@@ -36,7 +39,8 @@ class StepBatch:
         self.T = 0                      # tokens in the step
         self.R = 0                      # requests in the step
         self.token_ids = None           # [T]
-        self.positions = None           # [T] absolute position of each token in its request
+        self.positions = None           # [T] absolute position of each token in its request (what the cache and the attention count by)
+        self.position_axes = None       # [axes, T] positions for the encoding; with one axis, the same numbers
         self.seg_of_token = None        # [T] index of the token's request in this batch
         self.seg_offsets = None         # [R+1] prefix sums of new-token counts
         self.start_pos = None           # [R] tokens cached before this step
@@ -109,8 +113,12 @@ class StepRunner:
         replay.  `defer_copy`: the metadata stays in its staging buffer (`batch.pending_copy`): the
         caller fills in the token ids and sends it later.  `pad_rows` (steps of single tokens only):
         that many rows of no request follow the entries' rows, so that one recorded step serves every
-        number of requests up to its size: each is a token 0 at position 0 of a sequence of its own
-        whose only page is the cache's page for such rows; its logits are computed and not returned."""
+        number of requests up to its size: each is a token 0 at position 0 of a sequence of one token
+        whose only page is the cache's page for such rows; its logits are computed and not returned.
+        Such rows write their key and value to slot (row number mod page size) of that page: with more of
+        them than the page holds, several write the same slot in one launch, and all of them read key 0
+        of the page, which the first of them rewrites every step.  Harmless, because nothing of such a row
+        is ever returned and the page belongs to no request; no other page is touched."""
         cache = self.cache
         V = self.model.spec.vocab_size
         if not entries and not pad_rows:
@@ -133,6 +141,9 @@ class StepRunner:
             for t in e.tokens:
                 if not 0 <= t < V:
                     raise ValueError(f"request {e.req_id!r}: token id {t} is outside the vocabulary of {V}")
+            if e.positions is not None and (len(e.positions) != self.model.spec.position_axes
+                                            or any(len(ax) != n for ax in e.positions)):
+                raise ValueError(f"request {e.req_id!r}: positions must be [{self.model.spec.position_axes}][{n}]")
             if cache.length(e.req_id) + n > self.model.spec.max_positions:
                 raise ValueError(f"request {e.req_id!r}: {cache.length(e.req_id) + n} tokens exceed the model's "
                                  f"{self.model.spec.max_positions} positions")
@@ -177,7 +188,8 @@ class StepRunner:
             singles = []   # every token is single: the kernels take all rows
 
         # layout of the one int32 buffer
-        sizes = [("token_ids", T), ("positions", T), ("seg_of_token", T), ("seg_offsets", R + 1), ("start_pos", R),
+        axes = int(getattr(self.model.spec, "position_axes", 1))
+        sizes = [("token_ids", T), ("positions", T), ("axes", (axes if axes > 1 else 0) * T), ("seg_of_token", T), ("seg_offsets", R + 1), ("start_pos", R),
                  ("total_lens", R), ("want_rows", n_want), ("state_in", R), ("state_out", R),
                  ("att_tiles", len(tiles)), ("att_singles", len(singles))]
         for g in range(G):
@@ -208,6 +220,12 @@ class StepRunner:
                 a, b = offsets[i], offsets[i + 1]
                 pos[a:b] = np.arange(start[i], start[i] + lens[i])
                 sot[a:b] = i
+        if axes > 1:   # every axis the place in the sequence, unless the entry brings its own
+            ax = seg("axes").reshape(axes, T)
+            ax[:] = pos[None, :]
+            for i, e in enumerate(entries):
+                if e.positions is not None:
+                    ax[:, offsets[i]:offsets[i + 1]] = np.asarray(e.positions, dtype=np.int64)
         seg("seg_offsets")[:] = offsets
         seg("start_pos")[:] = start
         seg("total_lens")[:] = start + lens
@@ -270,6 +288,7 @@ class StepRunner:
         b = StepBatch()
         b.T, b.R = T, R
         b.token_ids, b.positions, b.seg_of_token = dseg("token_ids"), dseg("positions"), dseg("seg_of_token")
+        b.position_axes = dseg("axes").view(axes, T) if axes > 1 else b.positions.view(1, T)
         b.seg_offsets, b.start_pos, b.total_lens = dseg("seg_offsets"), dseg("start_pos"), dseg("total_lens")
         b.want_rows, b.state_in, b.state_out = dseg("want_rows"), dseg("state_in"), dseg("state_out")
         if tiles:
@@ -483,4 +502,5 @@ class StepRunner:
     def _graph_buffer_size(self, R: int, width: int) -> int:
         G = len(self.cache.groups)
         pad = lambda n: (n + 3) // 4 * 4
-        return 3 * pad(R) + pad(R + 1) + 5 * pad(R) + G * (pad(R) + pad(R * width)) + 64
+        axes = int(getattr(self.model.spec, "position_axes", 1))
+        return (3 + (axes if axes > 1 else 0)) * pad(R) + pad(R + 1) + 5 * pad(R) + G * (pad(R) + pad(R * width)) + 64

@@ -543,11 +543,15 @@ def bound_pages(need: int) -> int:
 
 def bound_rows(rows: int) -> int:
     """The number of rows a decode step of `rows` requests is served with when it is recorded: 1, 2, 4, 8,
-    16, 24, 32, 48, 64, 96, 128, ... (the rest are rows of no request).  The steps of these sizes stay within
-    the kernels' own row ranges (16, 32, 64 rows), so a filled-up step costs what the step itself would."""
-    b = 1
+    16, 24, 32, 48, 64, 96, 128, 160, 208, 256, 384, 512, ... (the rest are rows of no request).  The sizes end
+    where the products change kernels (16, 32, 64 rows; 208, the last size of the medium-rows product), so a
+    filled-up step runs the kernels the step itself would run and its recording equals the eager step."""
+    for b in (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 160, 208, 256):
+        if rows <= b:
+            return b
+    b = 256
     while b < rows:
-        b = b * 2 if b < 16 else (b * 3 // 2 if b & (b - 1) == 0 else b * 4 // 3)
+        b = b * 3 // 2 if b & (b - 1) == 0 else b * 4 // 3
     return b
 
 

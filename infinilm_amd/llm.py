@@ -85,9 +85,20 @@ class LLM:
         self.enable_graph = enable_graph
         if enable_graph and record_graphs_at_start:
             reach = model.spec.max_positions
-            if runner.cache.groups:   # no request holds more than the pool has
-                reach = min(reach, min(g.pool.num_pages for g in runner.cache.groups) * block_size)
+            if runner.cache.groups:
+                # no request holds more than the pool of the group that keeps all keys has (a group that keeps a
+                # window needs few pages however long the context: it does not bound the block table's width)
+                full = [g for g in runner.cache.groups if g.window <= 0] or runner.cache.groups
+                reach = min(reach, max(g.pool.num_pages for g in full) * block_size)
+            before = torch.cuda.memory_allocated()
             self.graphs_recorded_at_start = runner.record_decode_graphs(max_batch_size, reach)
+            self.graph_memory_bytes = torch.cuda.memory_allocated() - before
+            if self.graph_memory_bytes > (4 << 30):
+                import warnings
+                warnings.warn(f"the {self.graphs_recorded_at_start} decode recordings made at the start hold "
+                              f"{self.graph_memory_bytes / 2 ** 30:.1f} GiB of device memory (activations and logits of "
+                              "every size); lower max_batch_size or leave record_graphs_at_start off to record sizes as they come",
+                              RuntimeWarning)
         self.engine = LLMEngine(runner, max_num_seqs=max_batch_size, max_num_batched_tokens=max_num_batched_tokens,
                                 chunk_size=chunk_size, policy=admission, seed=seed, tokenizer=tokenizer,
                                 look_ahead=look_ahead)

@@ -419,6 +419,40 @@ def test_reserve_full_admission_never_runs_out_and_blocks_head_of_line():
     assert c.free_pages() == 8
 
 
+def test_reserve_full_counts_each_group_by_its_own_need():
+    """Two groups: one keeps all keys, one a window of 6 keys.  Full reservation asks of each group what a request
+    can hold there at most: all its pages in the first, the window's few in the second, so a small pool for the
+    windowed layers does not hold back requests that would never fill it; and no step ever runs out of pages."""
+    needs = [PagedKV(1, 4), PagedKV(1, 4, window=6)]
+    c = CacheManager(needs, page_size=4, num_pages=16, max_requests=6, dtype=torch.float32, device="cpu",
+                     num_pages_per_group={6: 9})
+    s = Scheduler(c, max_num_seqs=4, max_num_batched_tokens=16, chunk_size=4, policy="reserve_full", max_positions=1000)
+    assert s._group_pages(c.groups[0], 30) == 8 and s._group_pages(c.groups[1], 30) == 4   # window 6 + portion 4 -> 3 pages + 1
+    reqs = [_req("a", 20, max_tokens=10), _req("b", 18, max_tokens=12), _req("c", 5, max_tokens=3)]
+    for r in reqs:
+        s.add_request(r)
+    out = s.schedule()
+    # all keys: a and b need 8 pages each of 16; c waits for them (head of line).  With one need for all groups, b (8 pages)
+    # would not have fitted beside a in the windowed group's 9 pages.
+    assert [e.request.request_id for e in out.entries] == ["a", "b"]
+    for e in out.entries:
+        c.reserve(e.request.request_id, e.num_tokens); c.commit(e.request.request_id, e.num_tokens)
+    s.update(out, {})
+    peak = 0
+    for _ in range(200):
+        if not s.has_unfinished():
+            break
+        out = s.schedule()
+        for e in out.entries:
+            c.reserve(e.request.request_id, e.num_tokens)   # never OutOfPages
+            c.commit(e.request.request_id, e.num_tokens)
+        peak = max(peak, 9 - c.groups[1].pool.num_free)
+        s.update(out, {e.request.request_id: 7 for e in out.entries if e.samples})
+        c.check()
+    assert not s.has_unfinished() and s.num_preemptions == 0 and all(r.finish_reason == FinishReason.LENGTH for r in reqs)
+    assert peak <= 8 and c.groups[0].pool.num_free == 16 and c.groups[1].pool.num_free == 9
+
+
 def test_optimistic_admission_preempts_the_newest_when_pages_run_out():
     c = _cache(num_pages=6, page_size=4)
     s = Scheduler(c, max_num_seqs=4, max_num_batched_tokens=64, policy="optimistic", max_positions=1000)

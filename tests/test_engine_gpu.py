@@ -319,10 +319,47 @@ def test_recorded_steps_filled_up_with_rows_of_no_request(models):
                 r.cache.check()
     assert sizes == set(range(1, n + 1))
     assert {k[0] for k in graph._graphs} == {1, 2, 4, 8, 16}   # five recordings served eleven sizes
+    # the rows of no request wrote to the cache's spare page only: every page a request can hold equals the eager runner's
+    for e in eager.cache.k:
+        assert torch.equal(eager.cache.k[e][:48], graph.cache.k[e][:48]) and torch.equal(eager.cache.v[e][:48], graph.cache.v[e][:48])
     for r in (eager, graph):
         for rid in live:
             r.cache.release(rid)
         assert r.cache.free_pages() == 48
+
+
+@pytest.mark.parametrize("n,rows", [(17, 24), (33, 48), (65, 96), (129, 160), (161, 208)])
+def test_recorded_steps_filled_up_in_every_range_of_the_products(models, n, rows):
+    """17 requests run as 24 rows, 33 as 48, 65 as 96, 129 as 160, 161 as 208: one size in each range of rows in
+    which the products take another kernel (few rows with X in registers, 17 to 64, the medium-rows product up
+    to 208).  The recording, filled up with rows of no request, equals the eager step of the requests alone
+    bit for bit wherever the two run the same kernels, and within rounding where the filled-up step crosses
+    into the next kernel's range (the eager step of 17 rows and the recording of 24 both lie in one range)."""
+    from infinilm_amd import kernels
+    from infinilm_amd.engine.loading import load_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+
+    assert kernels.bound_rows(n) == rows
+    cfg, d, W = models[("B", "bfloat16")]
+    model = load_model(d, "bfloat16", "cuda:0")
+    eager = make_runner(model, num_pages=n + 8, page_size=16, max_requests=n)
+    graph = make_runner(model, num_pages=n + 8, page_size=16, max_requests=n, enable_graph=True)
+    graph.graph_after = 1
+    prompts = {f"r{i}": random_tokens(cfg, 1 + i % 7, 500 + i) for i in range(n)}
+    for r in (eager, graph):
+        for rid in prompts:
+            r.cache.admit(rid)
+        r.step([StepEntry(rid, p, []) for rid, p in prompts.items()])
+    nxt = {rid: 3 + i % 50 for i, rid in enumerate(prompts)}
+    for step in range(3):
+        entries = [StepEntry(rid, [nxt[rid]], [0]) for rid in prompts]
+        le = eager.step(entries).clone()
+        torch.cuda.synchronize()
+        lg = graph.step(entries)
+        assert lg.shape == le.shape
+        assert torch.equal(le.cpu(), lg.cpu()), f"{n} requests as {rows} rows, step {step}: replay differs from the eager step"
+        nxt = {rid: int(torch.argmax(le[i])) for i, rid in enumerate(prompts)}
+    assert {k[0] for k in graph._graphs} == {rows}
 
 
 def test_decode_steps_recorded_before_the_first_request(models):

@@ -546,6 +546,106 @@ def test_a_position_encoding_and_an_output_head_registered_from_outside(tmp_path
         drv.runner.step([StepEntry("c", [1] * (MAXP + 1), [])])
 
 
+def test_positions_over_two_axes_reach_a_position_encoding(tmp_path):
+    """A model whose spec says two position axes: the step carries [2, T] positions (every axis the place in the
+    sequence unless an entry brings its own), and a toy encoding defined here adds one learned table by axis 0 and
+    another by axis 1 to q and k.  Portions and decoded tokens of two requests, with columns that restart every
+    five tokens, against the plain formulas; the cache and the attention keep counting by the place in the sequence."""
+    from safetensors.torch import save_file
+    from infinilm_amd import kernels
+    from infinilm_amd.config import HeadSpec, LayerRun, LayerSpec, ModelSpec, PartSpec, register_architecture
+    from infinilm_amd.engine.loading import build_model, load_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+    from infinilm_amd.parts import Param, PositionEncoding, register_position_encoding
+
+    @register_position_encoding("toy_two_axes")
+    class ToyTwoAxes(PositionEncoding):
+        def __init__(self, head_dim, max_positions, ctx):
+            self.head_dim, self.max_positions = int(head_dim), int(max_positions)
+            self.rows = torch.empty((self.max_positions, self.head_dim), dtype=ctx.dtype, device=ctx.device)
+            self.cols = torch.empty((8, self.head_dim), dtype=ctx.dtype, device=ctx.device)
+            self._none = torch.zeros((1, 0), dtype=torch.float32, device=ctx.device)
+
+        def named_parameters(self):
+            return {"rows.weight": Param(self.rows), "cols.weight": Param(self.cols)}
+
+        def encode_and_store(self, qkv, batch, view, nh, nkv, d):
+            assert batch.position_axes.shape == (2, qkv.shape[0])
+            add = self.rows[batch.position_axes[0].long()] + self.cols[batch.position_axes[1].long()]
+            qkv[:, :(nh + nkv) * d].view(-1, nh + nkv, d).add_(add[:, None, :])
+            kernels.rope_kvwrite(qkv, batch.positions, self._none, self._none, view.k, view.v, view.slots, nh, nkv, d, 0)
+
+    H, d, nh, nkv, V, MAXP = 32, 16, 2, 1, 41, 64
+
+    def build_spec(cfg):
+        norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-6})
+        pos = PartSpec("toy_two_axes", {"head_dim": d, "max_positions": MAXP})
+        att = PartSpec("gqa_attention", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d, "qkv_bias": False,
+                                         "out_bias": False, "scale": d ** -0.5, "window": 0, "position": pos})
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 24, "bias": False})
+        names = {"norm1": "ln1", "mixer": "att", "norm2": "ln2", "ffn": "ffn"}
+        layers = [LayerSpec("l.0", "pre_norm", {"norm1": norm, "mixer": att, "norm2": norm, "ffn": ffn}, names, 1.0)]
+        return ModelSpec("ToyTwoAxesLM", V, H, MAXP, "emb", 1.0, layers, [LayerRun(0, 0)], norm, "ln_f", HeadSpec("head", 1.0, True),
+                         position_axes=2)
+
+    register_architecture(["ToyTwoAxesLM"], dict, build_spec)
+    mdir = str(tmp_path / "two_axes")
+    os.makedirs(mdir)
+    json.dump({"architectures": ["ToyTwoAxesLM"], "torch_dtype": "float32"}, open(os.path.join(mdir, "config.json"), "w"))
+    names = build_model({"architectures": ["ToyTwoAxesLM"]}, "float32", "meta").named_parameters()
+    g = torch.Generator().manual_seed(21)
+    W = {}
+    for name, p in sorted(names.items()):
+        if name == "head.weight":
+            continue
+        t = torch.randn(tuple(p.tensor.shape), generator=g) * 0.4
+        W[name] = (t * 0.25 + 1.0) if t.dim() == 1 else t
+    save_file(W, os.path.join(mdir, "model.safetensors"), metadata={"format": "pt"})
+    col = lambda i: i % 5
+
+    def plain(ids):
+        Wd = {k: v.to(F64) for k, v in W.items()}
+        n = len(ids)
+        x = Wd["emb.weight"][torch.tensor(ids)]
+        h = P.plain_rmsnorm(x, Wd["l.0.ln1.weight"], 1e-6)
+        off = (Wd["l.0.att.position.rows.weight"][:n] + Wd["l.0.att.position.cols.weight"][[col(i) for i in range(n)]])[:, None, :]
+        q = P.plain_linear(h, Wd["l.0.att.q_proj.weight"]).view(n, nh, d) + off
+        k = P.plain_linear(h, Wd["l.0.att.k_proj.weight"]).view(n, nkv, d) + off
+        v = P.plain_linear(h, Wd["l.0.att.v_proj.weight"]).view(n, nkv, d)
+        x = x + P.plain_linear(P.plain_attention(q, k, v, d ** -0.5).reshape(n, nh * d), Wd["l.0.att.o_proj.weight"])
+        h = P.plain_rmsnorm(x, Wd["l.0.ln2.weight"], 1e-6)
+        x = x + P.plain_mlp(h, Wd["l.0.ffn.gate_proj.weight"], Wd["l.0.ffn.up_proj.weight"], Wd["l.0.ffn.down_proj.weight"], 1.0)
+        return P.plain_linear(P.plain_rmsnorm(x, Wd["ln_f.weight"], 1e-6), Wd["emb.weight"])
+
+    model = load_model(mdir, "float32", "cuda:0")
+    r = make_runner(model, num_pages=12, page_size=8, max_requests=2)
+    g2 = torch.Generator().manual_seed(6)
+    a, b = (torch.randint(0, V, (n,), generator=g2).tolist() for n in (40, 13))
+    got = {"a": [], "b": []}
+
+    def step(parts):
+        es = []
+        for rid, toks, lo in parts:
+            if not r.cache.has(rid):
+                r.cache.admit(rid)
+            idx = list(range(lo, lo + len(toks)))
+            es.append(StepEntry(rid, toks, list(range(len(toks))), positions=[idx, [col(i) for i in idx]]))
+        out = r.step(es).cpu()
+        row = 0
+        for rid, toks, _ in parts:
+            got[rid].append(out[row:row + len(toks)].clone())
+            row += len(toks)
+
+    step([("a", a[:17], 0)])
+    step([("a", a[17:19], 17), ("b", b, 0)])
+    step([("a", a[19:20], 19)])
+    step([("a", a[20:], 20)])
+    assert rel_err(torch.cat(got["a"]), plain(a)) < 1e-4
+    assert rel_err(torch.cat(got["b"]), plain(b)) < 1e-4
+    with pytest.raises(ValueError, match=r"positions must be \[2\]"):
+        r.step([StepEntry("a", [1], [0], positions=[[40]])])
+
+
 def test_a_model_without_paged_keys_runs_through_the_entry_point_with_graphs(tmp_path):
     """Every mixer keeps a fixed-size state and none keeps pages: the scheduler's worst-case
     admission, the recorded decode steps and the look-ahead loop have no block table to lean on."""
