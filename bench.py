@@ -5,10 +5,11 @@
 A "step" is one decode step of the engine's own step function followed by greedy sampling, with
 `--batch` requests that each hold `--context` tokens in the paged cache when the last timed step
 ends.  One JSON line is printed: `value` is decoded tokens a second at the default batch;
-`prefill` is one 2,048-token prompt in one step; `roofline` prices the decode step against HBM
-bandwidth (every weight it uses read once, plus the cache of the live requests); `points` holds
-decode at batch 1, 32 and 64.  Peaks are MI355X's published ones (HBM 8 TB/s; dense MFMA bf16
-2.5 PFLOP/s, fp32 157.3 TFLOP/s).  Weights are random (N(0, 0.02), norms 1 + N(0, 0.02)) and the
+`prefill` is one 2,048-token prompt in one step (the median of seven passes timed with events);
+`roofline` prices the decode step against HBM bandwidth (every weight it uses read once, plus the
+cache of the live requests); `points` holds decode at batch 1, 32 and 64 and `points_frac` the same
+pricing of each; `fp32` the batch-8 step and the prefill on the true 32-bit path.  Peaks are MI355X's
+published ones (HBM 8 TB/s; dense MFMA bf16 2.5 PFLOP/s, fp32 157.3 TFLOP/s).  Weights are random (N(0, 0.02), norms 1 + N(0, 0.02)) and the
 cache of the context is filled with random keys and values instead of being computed: the timed
 steps do all of their work.
 """
@@ -47,7 +48,8 @@ def main() -> int:
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step eagerly")
     ap.add_argument("--prefill-only", action="store_true", help="only the prefill measurement (for profiling)")
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 32 / 64 points and the prefill")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 32 / 64 points, the prefill and the 32-bit record")
+    ap.add_argument("--no-fp32", action="store_true", help="skip the 32-bit record (bfloat16 runs only)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (N>1 is not run)")
@@ -55,24 +57,39 @@ def main() -> int:
 
     import torch
     from infinilm_amd.csrc import lib
-    from infinilm_amd.engine.loading import build_model, make_runner, require_gpu
-    from infinilm_amd.engine.step import StepEntry
-    from infinilm_amd.sampling import Sampler, SamplingParams
-    from infinilm_amd.weights import fill_random_
+    from infinilm_amd.engine.loading import require_gpu
 
     require_gpu("cuda:0")
     lib.load()
     FULL_LAYERS = 32
     cfg = config_8b(args.layers)
-    model = build_model(cfg, args.dtype, "cuda:0")
+    record = measure(args, cfg, args.dtype, FULL_LAYERS, full=True)
+    if args.dtype == "bfloat16" and not args.no_points and not args.no_fp32 and not args.prefill_only:
+        torch.cuda.empty_cache()
+        f = measure(args, cfg, "float32", FULL_LAYERS, full=False)
+        record["fp32"] = {"decode_b%d" % args.batch: f["value"], "ms_per_step": f["ms_per_step"], "hbm_frac": f["roofline"]["frac"],
+                          "prefill_ms": f["prefill"]["ms"], "prefill_frac": f["prefill"]["frac"]}
+    print(json.dumps(record))
+    return 0
+
+
+def measure(args, cfg, dtype, FULL_LAYERS, full):
+    """One dtype's record; `full`: with the batch 1 / 32 / 64 points."""
+    import torch
+    from infinilm_amd.engine.loading import build_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+    from infinilm_amd.sampling import Sampler, SamplingParams
+    from infinilm_amd.weights import fill_random_
+
+    model = build_model(cfg, dtype, "cuda:0")
     fill_random_(model, seed=0, std=0.02, norm_init="one_plus")
     torch.cuda.synchronize()
     spec = model.spec
     H, V, L = spec.hidden_size, spec.vocab_size, len(spec.order)
-    esize = 2 if args.dtype == "bfloat16" else 4
-    dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
+    esize = 2 if dtype == "bfloat16" else 4
+    dkey = "bf16" if dtype == "bfloat16" else "fp32"
 
-    max_b = max(args.batch, 1 if args.no_points else 64)
+    max_b = max(args.batch, 1 if (args.no_points or not full) else 64)
     ps = args.page_size
     pages_per_req = -(-(args.context + 1) // ps)
     num_pages = max(max_b * pages_per_req, -(-args.prefill_tokens // ps)) + 4
@@ -127,24 +144,26 @@ def main() -> int:
         T = args.prefill_tokens
         prompt = torch.randint(0, V, (T,), generator=gen).tolist()
         times = []
-        for i in range(3):
+        passes = 7 if dtype == "bfloat16" else 3
+        for i in range(passes + 1):   # the first pass warms up (the library chooses its kernels there)
             rid = f"p{i}"
             cache.admit(rid)
             torch.cuda.synchronize()
-            t0 = time.perf_counter()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
             logits = runner.step([StepEntry(rid, prompt, [T - 1])])
             sampler.sample(logits, [(greedy, 0, 0)])
+            e1.record()
             torch.cuda.synchronize()
-            times.append(time.perf_counter() - t0)
+            times.append(e0.elapsed_time(e1) * 1e-3)
             cache.release(rid)
-        pt = min(times[1:])
+        pt = sorted(times[1:])[len(times[1:]) // 2]   # the median
         mat_params = sum(t.numel() for t in inner if t.dim() == 2)
         flops = 2.0 * T * mat_params + 4.0 * T * T / 2.0 * cfg["num_attention_heads"] * cfg["head_dim"] * L + 2.0 * V * H
         return {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3), "frac": round(flops / pt / FLOP_PEAK[dkey], 4)}
 
     if args.prefill_only:
-        print(json.dumps({"prefill": prefill()}))
-        return 0
+        return {"prefill": prefill()}
     main_pt = decode(args.batch, args.steps, args.warmup)
     record = {
         "metric": "decode tokens/s, MiniCPM4-8B shape, batch %d, context %d" % (args.batch, args.context),
@@ -161,12 +180,14 @@ def main() -> int:
     }
     if not args.no_points:
         k = max(8, args.steps // 2)
-        record["points"] = {"decode_b1": round(decode(1, k, args.warmup)["tok_s"], 2),
-                            "decode_b32": round(decode(32, k, args.warmup)["tok_s"], 2),
-                            "decode_b64": round(decode(64, k, args.warmup)["tok_s"], 2)}
+        if full:
+            pts = {b: decode(b, k, args.warmup) for b in (1, 32, 64)}
+            record["points"] = {f"decode_b{b}": round(p["tok_s"], 2) for b, p in pts.items()}
+            # the same pricing as `roofline` for each point: bytes the step has to read / its time / the HBM peak
+            record["points_frac"] = {f"decode_b{b}": round(p["gbs"] * 1e9 / HBM_PEAK, 4) for b, p in pts.items()}
         record["prefill"] = prefill()
-    print(json.dumps(record))
-    return 0
+    del runner, cache, model
+    return record
 
 
 if __name__ == "__main__":

@@ -277,7 +277,11 @@ FEW_ROWS = int(os.environ.get("INFINILM_AMD_FEW_ROWS", "32"))
 
 
 def _few_rows(M: int, K: int) -> bool:
-    return M <= 16 or (M <= FEW_ROWS and K <= 4096)
+    """Whether the products that keep X in registers take M rows: a wave of eight holds the fragments of K / 8 of one
+    group of 16 rows in 4 registers a 32 k, and 256 registers take 16 rows of K up to 8192 or 32 rows of K up to 4096
+    beside the W fragments in flight."""
+    groups = max(1, min(FEW_ROWS // 16, 8192 // max(K, 4096)))
+    return M <= 16 * groups
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, alpha: float = 1.0,
@@ -309,7 +313,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     # at 160, 114 -> 48 at 192, 63 -> 51 at 208; o projection 22 -> 17, 25 -> 19, 32 -> 23 at 192)
     # (not for small matrices, whose few tiles leave most of the chip idle whatever the split: 0.5B shape at 128
     # rows 2.22 against 1.96 ms a step with the library)
-    if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS and N * K >= MID_MIN_WEIGHT:
+    if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS and _mid_fills_the_chip(N, K, a.device):
         return _gemm_mid(a, w, K, False)
     # 17 to 64 rows on their way into the residual sum: K in ranges of 1024 with the X fragments of all rows
     # in registers (o projection at 64 rows 13.1 against the library's 18.9 us, down projection 33.9
@@ -387,7 +391,15 @@ F32_FEW_ROWS = int(os.environ.get("INFINILM_AMD_F32_FEW_ROWS", "64"))
 ROWS64_SPAN = 1024   # K range of one part of the 17-to-64-rows product (ilm_gemm_rows64_span())
 ROWS64_MAX_PARTS = int(os.environ.get("INFINILM_AMD_ROWS64_PARTS", "16"))   # 0: never this kernel
 MID_MAX_ROWS = int(os.environ.get("INFINILM_AMD_MID_ROWS", "208"))  # 16: above 16 rows always the library
-MID_MIN_WEIGHT = 5 << 20   # elements of W from which the medium-rows product is used
+MID_MIN_WGS_PER_CU = 0.25   # the medium-rows product is used where its grid can give more than a quarter of the units a workgroup
+
+
+def _mid_fills_the_chip(N: int, K: int, device) -> bool:
+    """The medium-rows product cuts W into tiles of 128 rows and K into ranges of at least 512: with fewer
+    workgroups than a quarter of the compute units whatever the split, the vendor library's product is faster
+    (measured: the 0.5B shape's 1024 x 4096 gives 64 workgroups on 256 units and loses, 2.22 against 1.96 ms a step
+    at 128 rows; the 2B-family's 2304 x 2304 gives 72 and wins)."""
+    return -(-N // 128) * max(K // 512, 1) > MID_MIN_WGS_PER_CU * _num_cus(device)
 MID_TARGET_WGS = int(os.environ.get("INFINILM_AMD_MID_WGS", "512"))
 
 
