@@ -29,8 +29,9 @@ __device__ __forceinline__ f32x4 gw_mfma(uint4 a, uint4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-// MG: groups of 16 rows of X (2 to 4)
-template <int MG>
+// MG: groups of 16 rows of X (2 to 4).  FRAGW: W is given in fragment order (frag.h), tiles of 8 gate rows and the 8
+// up rows of the same outputs: a wave's W fragment is then 1 KB of consecutive bytes.
+template <int MG, bool FRAGW>
 __global__ void __launch_bounds__(GW_THREADS)
 gemm_gateup_wide_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W,
                         const bf16* __restrict__ bias, int M, int I, int K, int lda, int ldw, int ldc) {
@@ -50,7 +51,9 @@ gemm_gateup_wide_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const 
     // this lane's W row: rows 0..7 of the tile are gate rows, rows 8..15 the up rows of the same outputs
     // (clamped; outputs beyond I are never stored)
     const int nr = (n0 + (r & 7) < I) ? n0 + (r & 7) : I - 1;
-    const uint4* wp = reinterpret_cast<const uint4*>(W + (size_t)(nr + (r >> 3) * I) * ldw);
+    const int ksteps = (K + 31) >> 5;
+    const uint4* wp = FRAGW ? reinterpret_cast<const uint4*>(W) + (size_t)(blockIdx.x * GW_WAVES + wave) * ksteps * 64 + lane
+                            : reinterpret_cast<const uint4*>(W + (size_t)(nr + (r >> 3) * I) * ldw);
     // this thread's pieces of an X tile: k offset (tid % PR) * 8 of rows tid / PR + RPP i
     const int xk = threadIdx.x % PR, xr = threadIdx.x / PR;
     bf16* xs = &Xs[0][xr][xk * 8];
@@ -62,8 +65,13 @@ gemm_gateup_wide_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const 
     // access to that waits for all loads in flight.
 #define GW_LOAD_W(DST_, STEP_)                                                   \
     _Pragma("unroll") for (int s = 0; s < GW_KSUB; ++s) {                        \
-        const int k8 = (STEP_) * PR + s * 4 + q;                                 \
-        DST_[s] = wp[k8 <= k8_last ? k8 : k8_last];                              \
+        if (FRAGW) {                                                             \
+            const int st = (STEP_) * GW_KSUB + s;                                \
+            DST_[s] = wp[(size_t)(st < ksteps ? st : ksteps - 1) * 64];          \
+        } else {                                                                 \
+            const int k8 = (STEP_) * PR + s * 4 + q;                             \
+            DST_[s] = wp[k8 <= k8_last ? k8 : k8_last];                          \
+        }                                                                        \
     }
 #define GW_X1(XV_, I_)                                                           \
     if (XPER > I_) {                                                             \
@@ -165,20 +173,20 @@ gemm_gateup_wide_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const 
 
 // act [M, ldc] = silu(X Wg^T + bg) * (X Wu^T + bu) with W = [Wg; Wu] of 2 I rows (bias of 2 I entries or null),
 // 17 <= M <= 64 (made for 33 to 64: below, the kernels that keep X in registers are faster).
+// frag_w != 0: W is the weight in fragment order with tiles of 8 gate + 8 up rows (ldw is not used).
 extern "C" int ilm_gemm_gateup_wide(void* C, int ldc, const void* X, int lda, const void* W, int ldw, const void* bias,
-                                    int M, int I, int K, hipStream_t stream) {
+                                    int M, int I, int K, int frag_w, hipStream_t stream) {
     ILM_REQUIRE(M > 16 && M <= 64 && I > 0 && K > 0, "gemm_gateup_wide: needs 17 <= M <= 64, got M=%d I=%d K=%d", M, I, K);
-    ILM_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldc >= I,
+    ILM_REQUIRE(K % 8 == 0 && lda % 8 == 0 && (frag_w || (ldw % 8 == 0 && ldw >= K)) && lda >= K && ldc >= I,
                 "gemm_gateup_wide: K=%d lda=%d ldw=%d ldc=%d", K, lda, ldw, ldc);
     ILM_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_gateup_wide: operands must be 16-byte aligned");
     const int grid = (I + GW_NOUT - 1) / GW_NOUT;
     const bf16* b = (const bf16*)bias;
-    if (M <= 32)
-        gemm_gateup_wide_kernel<2><<<grid, GW_THREADS, 0, stream>>>((bf16*)C, (const bf16*)X, (const bf16*)W, b, M, I, K, lda, ldw, ldc);
-    else if (M <= 48)
-        gemm_gateup_wide_kernel<3><<<grid, GW_THREADS, 0, stream>>>((bf16*)C, (const bf16*)X, (const bf16*)W, b, M, I, K, lda, ldw, ldc);
-    else
-        gemm_gateup_wide_kernel<4><<<grid, GW_THREADS, 0, stream>>>((bf16*)C, (const bf16*)X, (const bf16*)W, b, M, I, K, lda, ldw, ldc);
+#define GW_GO(MG_)                                                                                                          \
+    if (frag_w) gemm_gateup_wide_kernel<MG_, true><<<grid, GW_THREADS, 0, stream>>>((bf16*)C, (const bf16*)X, (const bf16*)W, b, M, I, K, lda, ldw, ldc); \
+    else gemm_gateup_wide_kernel<MG_, false><<<grid, GW_THREADS, 0, stream>>>((bf16*)C, (const bf16*)X, (const bf16*)W, b, M, I, K, lda, ldw, ldc);
+    if (M <= 32) { GW_GO(2) } else if (M <= 48) { GW_GO(3) } else { GW_GO(4) }
+#undef GW_GO
     ILM_LAUNCH_CHECK("gemm_gateup_wide");
     return 0;
 }

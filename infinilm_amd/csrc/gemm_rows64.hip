@@ -23,6 +23,9 @@ __device__ __forceinline__ f32x4 r6_mfma(uint4 a, uint4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// FRAGW: W is given in fragment order (frag.h), tiles of 16 consecutive rows: a wave's W fragment is 1 KB of
+// consecutive bytes (a compute unit takes those in several times faster than fragments gathered from rows).
+template <bool FRAGW>
 __global__ void __launch_bounds__(R6_WAVES * 64)
 gemm_rows64_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W, int M, int N, int K,
                    int lda, int ldw, int ldc, size_t c_part_stride, int n_groups) {
@@ -43,8 +46,17 @@ gemm_rows64_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16
         k8c[u] = kok[u] ? k8 : k8_last;
     }
     const int ntiles = (N + 15) / 16;
+    const int ksteps = (K + 31) >> 5;
+    int wk[R6_KS];   // where a step's W fragment lies from the tile's (FRAGW) or the row's start, in 16-byte units
+#pragma unroll
+    for (int u = 0; u < R6_KS; ++u) wk[u] = FRAGW ? (k8c[u] >> 2) * 64 : k8c[u];
     // this lane's W row of tile t of a group (clamped: rows beyond N are never stored)
     auto w_row = [&](int group, int t) -> const uint4* {
+        if (FRAGW) {
+            int tile = group * R6_T + t;
+            tile = tile < ntiles ? tile : ntiles - 1;
+            return reinterpret_cast<const uint4*>(W) + (size_t)tile * ksteps * 64 + lane;
+        }
         int n = (group * R6_T + t) * 16 + r;
         n = n < N ? n : N - 1;
         return reinterpret_cast<const uint4*>(W + (size_t)n * ldw);
@@ -56,7 +68,7 @@ gemm_rows64_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16
         for (int t = 0; t < R6_T; ++t) {
             const uint4* wp = w_row(group, t);
 #pragma unroll
-            for (int u = 0; u < R6_KS; ++u) a[t][u] = wp[k8c[u]];
+            for (int u = 0; u < R6_KS; ++u) a[t][u] = wp[wk[u]];
         }
     }
     uint4 xf[R6_MG][R6_KS];
@@ -92,7 +104,7 @@ gemm_rows64_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16
             for (int t = 0; t < R6_T; ++t) {
                 const uint4* wp = w_row(next, t);
 #pragma unroll
-                for (int u = 0; u < R6_KS; ++u) a[t][u] = wp[k8c[u]];
+                for (int u = 0; u < R6_KS; ++u) a[t][u] = wp[wk[u]];
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -121,10 +133,11 @@ gemm_rows64_kernel(float* __restrict__ C, const bf16* __restrict__ X, const bf16
 extern "C" int ilm_gemm_rows64_span() { return R6_SPAN; }
 
 // C: float [kb][M][ldc] with c_part_stride elements between the parts, kb = ceil(K / ilm_gemm_rows64_span()).
+// frag_w != 0: W is the weight in fragment order, tiles of 16 consecutive rows (ldw is not used).
 extern "C" int ilm_gemm_rows64(void* C, int ldc, long c_part_stride, int kb, const void* W, int ldw, int M, int N, int K,
-                               const void* X, int lda, hipStream_t stream) {
+                               const void* X, int lda, int frag_w, hipStream_t stream) {
     ILM_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_rows64: needs 1 <= M <= 64, got M=%d N=%d K=%d", M, N, K);
-    ILM_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldc >= N,
+    ILM_REQUIRE(K % 8 == 0 && lda % 8 == 0 && (frag_w || (ldw % 8 == 0 && ldw >= K)) && lda >= K && ldc >= N,
                 "gemm_rows64: K=%d lda=%d ldw=%d ldc=%d", K, lda, ldw, ldc);
     ILM_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_rows64: operands must be 16-byte aligned");
     ILM_REQUIRE(kb == (K + R6_SPAN - 1) / R6_SPAN && kb <= 65535, "gemm_rows64: K=%d needs %d parts, got %d", K,
@@ -135,8 +148,12 @@ extern "C" int ilm_gemm_rows64(void* C, int ldc, long c_part_stride, int kb, con
     if (gx < 1) gx = 1;
     if (gx > n_groups) gx = n_groups;
     dim3 grid(gx, kb);
-    gemm_rows64_kernel<<<grid, R6_WAVES * 64, 0, stream>>>((float*)C, (const bf16*)X, (const bf16*)W, M, N, K, lda, ldw, ldc,
-                                                           (size_t)c_part_stride, n_groups);
+    if (frag_w)
+        gemm_rows64_kernel<true><<<grid, R6_WAVES * 64, 0, stream>>>((float*)C, (const bf16*)X, (const bf16*)W, M, N, K, lda, ldw,
+                                                                     ldc, (size_t)c_part_stride, n_groups);
+    else
+        gemm_rows64_kernel<false><<<grid, R6_WAVES * 64, 0, stream>>>((float*)C, (const bf16*)X, (const bf16*)W, M, N, K, lda, ldw,
+                                                                      ldc, (size_t)c_part_stride, n_groups);
     ILM_LAUNCH_CHECK("gemm_rows64");
     return 0;
 }

@@ -284,9 +284,14 @@ def _few_rows(M: int, K: int) -> bool:
     return M <= 16 * groups
 
 
+def _frag_of(frag_w):
+    """`frag_w` arguments are a FragWeight, a function that packs one when it is needed, or None."""
+    return frag_w() if callable(frag_w) else frag_w
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, alpha: float = 1.0,
          out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
-         allow_parts: bool = False) -> torch.Tensor:
+         allow_parts: bool = False, frag_w=None) -> torch.Tensor:
     """alpha * (a w^T + bias); a [M, K] with dense rows, w [N, K]; float accumulation.
 
     `allow_parts`: the result goes straight into the residual sum (add_rmsnorm), so it may come in
@@ -323,8 +328,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
             and -(-K // ROWS64_SPAN) <= ROWS64_MAX_PARTS and (M > FEW_ROWS or K <= KSPLIT_SPAN)):
         kb = -(-K // ROWS64_SPAN)
         parts = torch.empty((kb, M, N), dtype=F32, device=a.device)
-        _run("ilm_gemm_rows64", parts.data_ptr(), N, M * N, kb, w.data_ptr(), w.stride(0), M, N, K, a.data_ptr(),
-             a.stride(0), _stream())
+        fw = _frag_of(frag_w) if USE_FRAG else None
+        if fw is not None:   # W in fragment order: a wave's fragment is 1 KB of consecutive bytes
+            _run("ilm_gemm_rows64", parts.data_ptr(), N, M * N, kb, fw.data.data_ptr(), 0, M, N, K, a.data_ptr(),
+                 a.stride(0), 1, _stream())
+        else:
+            _run("ilm_gemm_rows64", parts.data_ptr(), N, M * N, kb, w.data_ptr(), w.stride(0), M, N, K, a.data_ptr(),
+                 a.stride(0), 0, _stream())
         return parts
     if fast and aligned and plain and allow_parts and out is None and M <= max(16, FEW_ROWS) and K > KSPLIT_SPAN and USE_KSPLIT:
         kb = -(-K // KSPLIT_SPAN)
@@ -473,7 +483,7 @@ def gateup_resident_ok(rows: int, w: torch.Tensor) -> bool:
 
 
 def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
-                       row_ss: Optional[torch.Tensor] = None, eps: float = 0.0) -> Optional[torch.Tensor]:
+                       row_ss: Optional[torch.Tensor] = None, eps: float = 0.0, frag_w=None) -> Optional[torch.Tensor]:
     """silu(x Wg^T + bg) * (x Wu^T + bu) for few rows in bfloat16, W = [Wg; Wu]: the fused gate/up
     projection with the SwiGLU in its epilogue, [M, I] (up to 32 rows with X in registers, up to 64 with X
     through LDS).  None where no kernel applies (more rows, float32): the caller then runs the projection
@@ -506,8 +516,13 @@ def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
         _run("ilm_gemm_gateup_swiglu", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
              _ptr(bias), M, I, K, _ptr(row_ss), 0 if row_ss is None else row_ss.shape[0], float(eps), _stream())
     else:
-        _run("ilm_gemm_gateup_wide", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
-             _ptr(bias), M, I, K, _stream())
+        fw = _frag_of(frag_w) if USE_FRAG else None
+        if fw is not None:   # W in fragment order (tiles of 8 gate + 8 up rows): 64.1 -> 56.8 us at 64 rows of the 8B shape
+            _run("ilm_gemm_gateup_wide", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), fw.data.data_ptr(), 0,
+                 _ptr(bias), M, I, K, 1, _stream())
+        else:
+            _run("ilm_gemm_gateup_wide", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
+                 _ptr(bias), M, I, K, 0, _stream())
     return out
 
 
@@ -779,6 +794,7 @@ def pack_weight(w: torch.Tensor, kind: str = "plain", **layout) -> FragWeight:
         raise KernelError("fragment order takes a bfloat16 weight with rows of a multiple of 8 elements, 16-byte aligned")
     N, K = w.shape
     rows = None
+    alloc_to = 4
     if kind == "plain":
         tiles = -(-N // 16)
     elif kind == "gate_up":
@@ -789,6 +805,15 @@ def pack_weight(w: torch.Tensor, kind: str = "plain", **layout) -> FragWeight:
         u = torch.where(idx < I, idx + I, torch.full_like(idx, -1))
         rows = torch.stack([g, u], dim=1).reshape(-1)
         tiles = 2 * it
+    elif kind == "gate_up8":   # tiles of 8 gate rows and the 8 up rows of the same outputs
+        I = N // 2
+        it = -(-I // 8)
+        idx = torch.arange(it * 8, dtype=torch.int64).view(it, 8)
+        g = torch.where(idx < I, idx, torch.full_like(idx, -1))
+        u = torch.where(idx < I, idx + I, torch.full_like(idx, -1))
+        rows = torch.cat([g, u], dim=1).reshape(-1)
+        tiles = it
+        alloc_to = 8   # a workgroup of the kernel that reads it takes 8 tiles
     elif kind == "qkv":
         nh, nkv, d = layout["nh"], layout["nkv"], layout["d"]
         half = d // 2
@@ -802,7 +827,7 @@ def pack_weight(w: torch.Tensor, kind: str = "plain", **layout) -> FragWeight:
         tiles = 2 * pt
     else:
         raise KernelError(f"unknown fragment layout {kind!r}")
-    alloc = -(-tiles // 4) * 4
+    alloc = -(-tiles // alloc_to) * alloc_to
     steps = -(-K // 32)
     data = torch.zeros((alloc * steps * 64 * 4,), dtype=torch.int32, device=w.device)
     rows_dev = None

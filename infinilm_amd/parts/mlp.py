@@ -34,7 +34,8 @@ class SwiGLU(FeedForward):
         if isinstance(x, DeferredNorm):   # the norm's division happens in the gate/up kernel's epilogue
             act = kernels.gateup_swiglu_gemm(x.x, self.gate_up.weight, self.gate_up.bias, row_ss=x.sumsq, eps=x.eps)
             return self.down.forward(act, allow_parts=True)
-        act = kernels.gateup_swiglu_gemm(x, self.gate_up.weight, self.gate_up.bias)   # few rows: activation in the epilogue
+        frag = (lambda: self.gate_up.frag_weight("gate_up8")) if kernels.frag_weight_ok(self.gate_up.weight) else None
+        act = kernels.gateup_swiglu_gemm(x, self.gate_up.weight, self.gate_up.bias, frag_w=frag)   # few rows: activation in the epilogue
         if act is not None:
             return self.down.forward(act, allow_parts=True)
         gu = self.gate_up.forward(x)

@@ -224,10 +224,11 @@ def test_gemm_bfloat16(K, M, N, K_, out_dtype):
 def test_gemm_split_over_k_and_its_consumer(K, monkeypatch, M, N, K_):
     """Few rows and long K: the product comes as float32 parts; add_rmsnorm sums them in order."""
     a, w = _rand((M, K_), 14, torch.bfloat16), _rand((N, K_), 15, torch.bfloat16, 0.05)
-    if M > 64 and N * K_ < K.MID_MIN_WEIGHT:
+    small = M > 64 and not K._mid_fills_the_chip(N, K_, torch.device(DEV))
+    if small:
         # a small matrix is left to the library on the engine's path; the medium-rows kernel is tested all the same
         assert K.gemm(a.to(DEV), w.to(DEV), allow_parts=True).dtype == torch.bfloat16
-        monkeypatch.setattr(K, "MID_MIN_WEIGHT", 0)
+        monkeypatch.setattr(K, "MID_MIN_WGS_PER_CU", -1.0)
     parts = K.gemm(a.to(DEV), w.to(DEV), allow_parts=True)
     if 16 < M <= 64 and K_ % 8 == 0:   # K ranges of 1024 (up to 32 rows with K beyond 4096: ranges of 4096)
         assert parts.shape[0] == (-(-K_ // 4096) if M <= 32 and K_ > 4096 else -(-K_ // 1024))
@@ -245,7 +246,7 @@ def test_gemm_split_over_k_and_its_consumer(K, monkeypatch, M, N, K_):
     short = K.gemm(a[:, :256].contiguous().to(DEV), w[:, :256].contiguous().to(DEV), allow_parts=True)
     # short K: float32, not rounded to bfloat16 (more than 16 rows: parts)
     # (many rows of a small matrix: the library's bfloat16 result)
-    assert (short.dtype == torch.float32 and short.dim() == 2) if M <= 16 else (short.dim() == 3 or (M > 64 and N * 256 < K.MID_MIN_WEIGHT))
+    assert (short.dtype == torch.float32 and short.dim() == 2) if M <= 16 else (short.dim() == 3 or M > 64)
     _close(whole, want, 6e-3)
     r = _rand((M, N), 16, scale=2.0)
     nw = _rand((N,), 17, torch.bfloat16) + 1
