@@ -429,6 +429,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
     const int tile_id = gridDim.x - 1 - item / gridDim.y;
     const int by = item % gridDim.y;
     const int t0 = tiles[2 * tile_id], ntok = tiles[2 * tile_id + 1];
+    if (ntok <= 0) return;   // a tile of no tokens: what fills up the list of a recorded step (the whole workgroup leaves)
     const int G = nh / nkv;
     const int HG = (G + 15) / 16;
     const int kvh = by / HG, hg = by % HG;

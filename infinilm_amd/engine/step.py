@@ -78,6 +78,10 @@ class StepRunner:
         self._graph_pool = None
         self._graph_seen: Dict = {}      # sizes met in eager steps so far -> how often
         self.graph_after = 2
+        # steps with portions of prompts are recorded too, by their bounded shape, where every layer's parts say that they
+        # take their indices from the device's tensors in such steps
+        self.graph_mixed = all(getattr(b, "records_mixed_steps", False) for b in getattr(model, "blocks", []))
+        self.graph_mixed_max_tokens = 8192   # ... up to this many tokens a step (a recording keeps the step's activations)
         self._pinned: List[Optional[torch.Tensor]] = [None, None]   # two staging buffers in turn
         self._copy_done: List[Optional[torch.cuda.Event]] = [None, None]
         self._stage_turn = 0
@@ -105,7 +109,7 @@ class StepRunner:
 
     def build_batch(self, entries: Sequence[StepEntry], min_blocks: int = 0,
                     device_buffer: Optional[torch.Tensor] = None, defer_copy: bool = False,
-                    pad_rows: int = 0) -> StepBatch:
+                    pad_rows: int = 0, bounds: Optional[tuple] = None) -> StepBatch:
         """Reserves pages for every entry and lays the step's metadata out.
 
         `min_blocks` pads the block tables to a fixed width and `device_buffer` receives the
@@ -118,7 +122,11 @@ class StepRunner:
         Such rows write their key and value to slot (row number mod page size) of that page: with more of
         them than the page holds, several write the same slot in one launch, and all of them read key 0
         of the page, which the first of them rewrites every step.  Harmless, because nothing of such a row
-        is ever returned and the page belongs to no request; no other page is touched."""
+        is ever returned and the page belongs to no request; no other page is touched.
+        `bounds` = (requests, wanted rows, attention tiles, single rows): every array of the metadata is laid out
+        for that many entries (with `pad_rows` and `min_blocks` for the tokens and the block tables), so that a
+        recorded step of mixed content finds every array at the same address at every replay: lists are
+        filled up with entries that do nothing (tiles of no tokens, a single row or a wanted row once more)."""
         cache = self.cache
         V = self.model.spec.vocab_size
         if not entries and not pad_rows:
@@ -158,11 +166,16 @@ class StepRunner:
             raise
 
         R_real = len(entries)
-        if pad_rows and any(len(e.tokens) != 1 for e in entries):
+        if pad_rows and bounds is None and any(len(e.tokens) != 1 for e in entries):
             raise ValueError("rows of no request fill up steps of single tokens only")
-        R = R_real + int(pad_rows)
+        # rows of no request: a sequence of one token each after decoded tokens; after a mixed step's tokens
+        # (bounded layout) one segment that holds them all, every one at position 0
+        pad_segs = int(pad_rows) if bounds is None else (1 if pad_rows else 0)
+        R = R_real + pad_segs
         lens = np.ones(R, dtype=np.int64)
         lens[:R_real] = [len(e.tokens) for e in entries]
+        if bounds is not None and pad_rows:
+            lens[R_real] = int(pad_rows)
         T = int(lens.sum())
         start = np.zeros(R, dtype=np.int64)
         start[:R_real] = [cache.length(e.req_id) for e in entries]
@@ -171,7 +184,7 @@ class StepRunner:
         G = len(cache.groups)
         ps = cache.page_size
         max_blocks = [max(1, min_blocks, max((len(cache.table(e.req_id, g)) for e in entries), default=0)) for g in range(G)]
-        n_want = sum(len(e.want) for e in entries) + int(pad_rows)
+        n_want = sum(len(e.want) for e in entries) + (int(pad_rows) if bounds is None else 0)
 
         # attention work lists: runs of up to TILE consecutive tokens of a request, and single tokens
         TILE = kernels.ATT_TILE_TOKENS
@@ -186,15 +199,21 @@ class StepRunner:
                     tiles += [a + k, min(TILE, n - k)]
         if not tiles:
             singles = []   # every token is single: the kernels take all rows
+        # (the rows of no request of a bounded layout are left out of the attention: nothing reads what they hold)
+        R_lay, want_lay, tiles_lay, singles_lay = R, n_want, len(tiles) // 2, len(singles)
+        if bounds is not None:
+            R_lay, want_lay, tiles_lay, singles_lay = bounds
+            if R > R_lay or n_want > want_lay or len(tiles) // 2 > tiles_lay or len(singles) > singles_lay or not tiles:
+                raise RuntimeError("a step does not fit the bounds it is laid out for")
 
         # layout of the one int32 buffer
         axes = int(getattr(self.model.spec, "position_axes", 1))
-        sizes = [("token_ids", T), ("positions", T), ("axes", (axes if axes > 1 else 0) * T), ("seg_of_token", T), ("seg_offsets", R + 1), ("start_pos", R),
-                 ("total_lens", R), ("want_rows", n_want), ("state_in", R), ("state_out", R),
-                 ("att_tiles", len(tiles)), ("att_singles", len(singles))]
+        sizes = [("token_ids", T), ("positions", T), ("axes", (axes if axes > 1 else 0) * T), ("seg_of_token", T), ("seg_offsets", R_lay + 1), ("start_pos", R_lay),
+                 ("total_lens", R_lay), ("want_rows", want_lay), ("state_in", R_lay), ("state_out", R_lay),
+                 ("att_tiles", 2 * tiles_lay), ("att_singles", singles_lay)]
         for g in range(G):
             sizes.append((f"slots{g}", T))
-            sizes.append((f"bt{g}", R * max_blocks[g]))
+            sizes.append((f"bt{g}", R_lay * max_blocks[g]))
         off = {}
         total = 0
         for name, n in sizes:
@@ -218,7 +237,7 @@ class StepRunner:
         else:
             for i in range(R):
                 a, b = offsets[i], offsets[i + 1]
-                pos[a:b] = np.arange(start[i], start[i] + lens[i])
+                pos[a:b] = np.arange(start[i], start[i] + lens[i]) if i < R_real else 0
                 sot[a:b] = i
         if axes > 1:   # every axis the place in the sequence, unless the entry brings its own
             ax = seg("axes").reshape(axes, T)
@@ -226,20 +245,30 @@ class StepRunner:
             for i, e in enumerate(entries):
                 if e.positions is not None:
                     ax[:, offsets[i]:offsets[i + 1]] = np.asarray(e.positions, dtype=np.int64)
-        seg("seg_offsets")[:] = offsets
-        seg("start_pos")[:] = start
-        seg("total_lens")[:] = start + lens
+        seg("seg_offsets")[:R + 1] = offsets
+        seg("seg_offsets")[R + 1:] = T
+        seg("start_pos")[:R] = start
+        seg("start_pos")[R:] = 0
+        seg("total_lens")[:R] = start + lens
+        seg("total_lens")[R_real:] = 1
         w = seg("want_rows")
         k = 0
         for i, e in enumerate(entries):
             for x in e.want:
                 w[k] = offsets[i] + x
                 k += 1
-        for i in range(R_real, R):
-            w[k] = offsets[i]
-            k += 1
-        seg("att_tiles")[:] = tiles
-        seg("att_singles")[:] = singles
+        if bounds is None:
+            for i in range(R_real, R):
+                w[k] = offsets[i]
+                k += 1
+        w[k:] = w[k - 1] if k else 0   # (a bounded layout: the last wanted row once more)
+        at = seg("att_tiles")
+        at[:len(tiles)] = tiles
+        at[len(tiles):] = 0             # tiles of no tokens
+        asg = seg("att_singles")
+        asg[:len(singles)] = singles
+        if singles_lay > len(singles):   # a row of no request, or the last single row once more (the same result written again)
+            asg[len(singles):] = int(offsets[R_real]) if pad_rows else singles[-1]
         sin, sout = seg("state_in"), seg("state_out")
         for i, e in enumerate(entries):
             sin[i], sout[i] = cache.state_rows(e.req_id)
@@ -247,7 +276,7 @@ class StepRunner:
         sout[R_real:] = cache.null_state_row
         for g in range(G):
             sl = seg(f"slots{g}")
-            bt = seg(f"bt{g}").reshape(R, max_blocks[g])
+            bt = seg(f"bt{g}").reshape(R_lay, max_blocks[g])
             bt[:] = -1
             if all_single:
                 slot_list = []
@@ -271,6 +300,9 @@ class StepRunner:
                 if (pages < 0).any():
                     raise RuntimeError(f"request {e.req_id!r}: a new token falls on a page already given back")
                 sl[offsets[i]:offsets[i + 1]] = pages * ps + p % ps
+            if pad_rows:   # rows of no request after a mixed step's tokens
+                bt[R_real:R, 0] = cache.null_page(g)
+                sl[offsets[R_real]:] = cache.null_page(g) * ps + np.arange(pad_rows) % ps
 
         if device_buffer is None:
             dev = torch.empty((total,), dtype=torch.int32, device=self.device)
@@ -291,14 +323,16 @@ class StepRunner:
         b.position_axes = dseg("axes").view(axes, T) if axes > 1 else b.positions.view(1, T)
         b.seg_offsets, b.start_pos, b.total_lens = dseg("seg_offsets"), dseg("start_pos"), dseg("total_lens")
         b.want_rows, b.state_in, b.state_out = dseg("want_rows"), dseg("state_in"), dseg("state_out")
+        b.layout_size = total
         if tiles:
             b.att_tiles = dseg("att_tiles").view(-1, 2)
-            b.att_single_rows = dseg("att_singles") if singles else None
-        b.block_tables = [dseg(f"bt{g}").view(R, max_blocks[g]) for g in range(G)]
+            b.att_single_rows = dseg("att_singles") if singles_lay else None
+        b.block_tables = [dseg(f"bt{g}").view(R_lay, max_blocks[g]) for g in range(G)]
         b.slots = [dseg(f"slots{g}") for g in range(G)]
-        b.num_wanted = n_want
+        b.num_wanted = want_lay
         b.rows_of_requests = T - int(pad_rows)   # the rows after them belong to no request
-        b.wants_all_rows = n_want == T and all(list(e.want) == list(range(len(e.tokens))) for e in entries)
+        b.wants_all_rows = (bounds is None and n_want == T
+                            and all(list(e.want) == list(range(len(e.tokens))) for e in entries))
         b.max_q_len = int(lens.max())
         b.max_total_len = int((start + lens).max())
         b.max_position = b.max_total_len - 1
@@ -325,6 +359,13 @@ class StepRunner:
                 self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
             if key in self._graphs or self._graph_seen[key] >= self.graph_after:
                 return self._graph_step(entries, key)
+        elif self.enable_graph and self.graph_mixed and taps is None and any(len(e.tokens) > 1 for e in entries):
+            key = self._mixed_key(entries)
+            if key is not None:
+                if key not in self._graphs:
+                    self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
+                if key in self._graphs or self._graph_seen[key] >= self.graph_after:
+                    return self._mixed_graph_step(entries, key)
         batch = self.build_batch(entries)
         batch.taps = taps
         logits = self.model.forward(batch, self.cache)
@@ -382,6 +423,65 @@ class StepRunner:
         self.tokens += R
         self._prepare_next_decode(entries)
         return logits[:R]
+
+    # ---- steps with portions of prompts as captured graphs -------------------------------------------
+    def _mixed_key(self, entries: Sequence[StepEntry]):
+        """The bounded shape of a step that holds portions of prompts (and decoded tokens beside them): tokens, requests,
+        wanted rows and block-table width, each rounded up (`kernels.bound_rows`, `kernels.bound_pages`); the lists of
+        attention tiles and of single rows are as long as those allow.  Under a token budget the steps of a busy engine have the budget's tokens and differ in
+        the rest by little, so few shapes serve them.  None: not recorded (too many tokens)."""
+        cache = self.cache
+        TILE = kernels.ATT_TILE_TOKENS
+        T = sum(len(e.tokens) for e in entries)
+        if T > self.graph_mixed_max_tokens:
+            return None
+        T_b = kernels.bound_rows(T)
+        R_b = kernels.bound_rows(len(entries) + 1)
+        n_want = sum(len(e.want) for e in entries)
+        need = max(-(-(cache.length(e.req_id) + len(e.tokens)) // cache.page_size) for e in entries)
+        # tiles and single rows need no bound of their own: at most a tile every TILE tokens and one more a request;
+        # at most a single row a request (none at all where no request brings one token and no row is filled up)
+        singles = any(len(e.tokens) == 1 for e in entries) or T_b > T
+        return ("mixed", T_b, R_b, kernels.bound_rows(max(n_want, 1)), T_b // TILE + R_b, R_b if singles else 0,
+                kernels.bound_pages(need))
+
+    def _mixed_graph_step(self, entries: Sequence[StepEntry], key) -> torch.Tensor:
+        """Replays (or first records) the step of bounded shape `key` with the entries' tokens first and rows of no
+        request after them; only the metadata buffer changes between replays."""
+        _, T_b, R_b, want_b, tiles_b, singles_b, width = key
+        T = sum(len(e.tokens) for e in entries)
+        n_want = sum(len(e.want) for e in entries)
+        self._prepared = None
+        slot = self._graphs.get(key)
+        build = lambda buf: self.build_batch(entries, min_blocks=width, device_buffer=buf, pad_rows=T_b - T,
+                                             bounds=(R_b, want_b, tiles_b, singles_b))
+        if slot is None:
+            probe = self.build_batch(entries, min_blocks=width, pad_rows=T_b - T, bounds=(R_b, want_b, tiles_b, singles_b),
+                                     defer_copy=True)   # (pages are reserved here; the layout's size is what is wanted)
+            buf = torch.zeros((probe.layout_size + 64,), dtype=torch.int32, device=self.device)
+            batch = build(buf)
+            batch.max_total_len = width * self.cache.page_size
+            saved = self.cache.snapshot_states([e.req_id for e in entries])
+            self.model.forward(batch, self.cache)      # warm-up outside the capture; the replay writes the same keys again
+            self.cache.restore_states(saved)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                logits = self.model.forward(batch, self.cache)
+            self._graphs[key] = (graph, batch, logits, buf)
+        else:
+            graph, batch, logits, buf = slot
+            fresh = build(buf)
+            if fresh.T != batch.T or fresh.layout_size != batch.layout_size:
+                raise RuntimeError("a step does not fit the graph captured for its shape")
+        graph.replay()
+        for e in entries:
+            self.cache.commit(e.req_id, len(e.tokens), e.tokens)
+        self.steps += 1
+        self.tokens += T
+        return logits[:n_want]
 
     def _record(self, key, entries: Sequence[StepEntry]):
         """Records the decode step of size `key` with the entries' rows first and rows of no request

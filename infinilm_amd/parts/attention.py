@@ -47,6 +47,7 @@ class GQAttention(Mixer):
         return PagedKV(self.nkv, self.d, self.window)
 
     takes_tail = True
+    records_mixed_steps = True
 
     def takes_frag(self, rows: int) -> bool:
         fn = getattr(self.position, "takes_frag", None)

@@ -107,6 +107,9 @@ class Norm(Part):
 class Mixer(Part):
     """`takes_tail`: forward accepts `tail=NormTail` and may answer with a DeferredNorm."""
     takes_tail = False
+    # True: forward takes every index from the batch's device tensors also in steps that hold portions of prompts
+    # (never from the host copies `h_*`), so that such steps can be recorded and replayed for other requests
+    records_mixed_steps = False
 
     def takes_frag(self, rows: int) -> bool:
         """Whether forward accepts x as `kernels.FragRows` (rows in fragment order) for a step of `rows` rows."""
@@ -120,6 +123,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    records_mixed_steps = False   # as for a mixer: nothing in forward depends on the host's view of the batch
+
     def takes_deferred(self, rows: int) -> bool:
         """Whether forward accepts a DeferredNorm of `rows` rows as x."""
         return False

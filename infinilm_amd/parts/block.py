@@ -36,6 +36,10 @@ class PreNormBlock:
     def cache_need(self):
         return self.mixer.cache_need()
 
+    @property
+    def records_mixed_steps(self) -> bool:
+        return bool(getattr(self.mixer, "records_mixed_steps", False) and getattr(self.ffn, "records_mixed_steps", False))
+
     def forward(self, stream: ResidualStream, batch, cache_view) -> None:
         # a decode step of many rows: the mixer may take its rows in fragment order, which the norm then writes
         rows = stream.residual.shape[0]

@@ -17,6 +17,8 @@ from .registry import register_feed_forward
 
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
+    records_mixed_steps = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, bias: bool, ctx: BuildContext):
         self.gate_up = FusedLinear(hidden_size, [intermediate_size, intermediate_size], ["gate_proj", "up_proj"],
                                    bias, ctx)
