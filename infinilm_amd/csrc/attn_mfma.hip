@@ -58,6 +58,7 @@ attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __re
     __shared__ float sm_acc[ATT_WAVES][D16][64][4];
     __shared__ float sm_ml[ATT_WAVES][16][2];
     const int t = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
+    if (t < 0) return;   // an entry that fills up the list of a recorded step: no row (the whole workgroup leaves)
     const int G = nh / nkv;
     const int HG = (G + 15) / 16;
     const int kvh = blockIdx.y / HG, hg = blockIdx.y % HG;
@@ -241,6 +242,7 @@ attn_merge_one_wave_kernel(bf16* __restrict__ out, const float* __restrict__ ws_
                   int window, int nsplit, int span) {
     __shared__ float wsm[64];
     const int t = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
+    if (t < 0) return;   // an entry that fills up the list of a recorded step: no row (the whole workgroup leaves)
     const int h = blockIdx.y, lane = threadIdx.x;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
@@ -307,6 +309,7 @@ attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws_acc, cons
     __shared__ float red[2][ATT_MERGE_WAVES];
     __shared__ float part[ATT_MERGE_WAVES][256];
     const int t = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
+    if (t < 0) return;   // an entry that fills up the list of a recorded step: no row (the whole workgroup leaves)
     const int h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;

@@ -131,6 +131,8 @@ class StepRunner:
         V = self.model.spec.vocab_size
         if not entries and not pad_rows:
             raise ValueError("a step needs at least one entry")
+        if not entries:
+            min_blocks = max(min_blocks, 1)
         if not defer_copy:
             # prepared metadata lies in one of the two staging buffers that this step and the next take
             # in turn: it does not outlive a step built in between
@@ -197,13 +199,13 @@ class StepRunner:
             else:
                 for k in range(0, n, TILE):
                     tiles += [a + k, min(TILE, n - k)]
-        if not tiles:
+        if not tiles and bounds is None:
             singles = []   # every token is single: the kernels take all rows
         # (the rows of no request of a bounded layout are left out of the attention: nothing reads what they hold)
         R_lay, want_lay, tiles_lay, singles_lay = R, n_want, len(tiles) // 2, len(singles)
         if bounds is not None:
             R_lay, want_lay, tiles_lay, singles_lay = bounds
-            if R > R_lay or n_want > want_lay or len(tiles) // 2 > tiles_lay or len(singles) > singles_lay or not tiles:
+            if R > R_lay or n_want > want_lay or len(tiles) // 2 > tiles_lay or len(singles) > singles_lay:
                 raise RuntimeError("a step does not fit the bounds it is laid out for")
 
         # layout of the one int32 buffer
@@ -261,14 +263,13 @@ class StepRunner:
             for i in range(R_real, R):
                 w[k] = offsets[i]
                 k += 1
-        w[k:] = w[k - 1] if k else 0   # (a bounded layout: the last wanted row once more)
+        w[k:] = w[k - 1] if k else T - 1   # (a bounded layout: the last wanted row once more)
         at = seg("att_tiles")
         at[:len(tiles)] = tiles
         at[len(tiles):] = 0             # tiles of no tokens
         asg = seg("att_singles")
         asg[:len(singles)] = singles
-        if singles_lay > len(singles):   # a row of no request, or the last single row once more (the same result written again)
-            asg[len(singles):] = int(offsets[R_real]) if pad_rows else singles[-1]
+        asg[len(singles):] = -1         # no row: the kernels skip such entries
         sin, sout = seg("state_in"), seg("state_out")
         for i, e in enumerate(entries):
             sin[i], sout[i] = cache.state_rows(e.req_id)
@@ -324,7 +325,7 @@ class StepRunner:
         b.seg_offsets, b.start_pos, b.total_lens = dseg("seg_offsets"), dseg("start_pos"), dseg("total_lens")
         b.want_rows, b.state_in, b.state_out = dseg("want_rows"), dseg("state_in"), dseg("state_out")
         b.layout_size = total
-        if tiles:
+        if tiles or bounds is not None:
             b.att_tiles = dseg("att_tiles").view(-1, 2)
             b.att_single_rows = dseg("att_singles") if singles_lay else None
         b.block_tables = [dseg(f"bt{g}").view(R_lay, max_blocks[g]) for g in range(G)]
@@ -431,19 +432,24 @@ class StepRunner:
         attention tiles and of single rows are as long as those allow.  Under a token budget the steps of a busy engine have the budget's tokens and differ in
         the rest by little, so few shapes serve them.  None: not recorded (too many tokens)."""
         cache = self.cache
-        TILE = kernels.ATT_TILE_TOKENS
         T = sum(len(e.tokens) for e in entries)
         if T > self.graph_mixed_max_tokens:
             return None
-        T_b = kernels.bound_rows(T)
-        R_b = kernels.bound_rows(len(entries) + 1)
         n_want = sum(len(e.want) for e in entries)
         need = max(-(-(cache.length(e.req_id) + len(e.tokens)) // cache.page_size) for e in entries)
-        # tiles and single rows need no bound of their own: at most a tile every TILE tokens and one more a request;
-        # at most a single row a request (none at all where no request brings one token and no row is filled up)
-        singles = any(len(e.tokens) == 1 for e in entries) or T_b > T
-        return ("mixed", T_b, R_b, kernels.bound_rows(max(n_want, 1)), T_b // TILE + R_b, R_b if singles else 0,
-                kernels.bound_pages(need))
+        return self._mixed_shape(kernels.bound_rows(T), n_want, any(len(e.tokens) == 1 for e in entries), need)
+
+    def _mixed_shape(self, T_b: int, n_want: int, singles: bool, pages: int):
+        """The key of a bounded shape.  Requests: as many as the cache takes, and one segment for the rows of no request
+        (the lists they size are small; a bound that followed the step's own number would multiply the shapes).  Wanted
+        rows: one a request, more if the step asks for more.  Tiles: at most one every TILE tokens and one more a request.
+        Single rows: one a request, or none.  Block-table width: a power of two."""
+        R_b = kernels.bound_rows(self.cache.max_requests + 1)
+        width = 4
+        while width < pages:
+            width *= 2
+        return ("mixed", T_b, R_b, max(R_b, kernels.bound_rows(max(n_want, 1))), T_b // kernels.ATT_TILE_TOKENS + R_b,
+                R_b if singles else 0, width)
 
     def _mixed_graph_step(self, entries: Sequence[StepEntry], key) -> torch.Tensor:
         """Replays (or first records) the step of bounded shape `key` with the entries' tokens first and rows of no
@@ -451,6 +457,8 @@ class StepRunner:
         _, T_b, R_b, want_b, tiles_b, singles_b, width = key
         T = sum(len(e.tokens) for e in entries)
         n_want = sum(len(e.want) for e in entries)
+        if len(entries) + 1 > R_b:
+            raise RuntimeError("more requests in a step than the cache takes")
         self._prepared = None
         slot = self._graphs.get(key)
         build = lambda buf: self.build_batch(entries, min_blocks=width, device_buffer=buf, pad_rows=T_b - T,
@@ -476,12 +484,36 @@ class StepRunner:
             fresh = build(buf)
             if fresh.T != batch.T or fresh.layout_size != batch.layout_size:
                 raise RuntimeError("a step does not fit the graph captured for its shape")
+        if not entries:
+            return logits[:0]    # a recording made ahead of the requests
         graph.replay()
         for e in entries:
             self.cache.commit(e.req_id, len(e.tokens), e.tokens)
         self.steps += 1
         self.tokens += T
         return logits[:n_want]
+
+    def record_mixed_graphs(self, tokens: int, max_context: int) -> int:
+        """Records, before any request has come, the steps of `tokens` tokens (a full token budget) with portions of
+        prompts, with and without decoded tokens beside them, for every block-table width up to `max_context` tokens:
+        returns how many were made."""
+        if not (self.enable_graph and self.graph_mixed) or tokens < 2 or tokens > self.graph_mixed_max_tokens:
+            return 0
+        made = 0
+        pages = max(1, -(-int(max_context) // self.cache.page_size)) if self.cache.groups else 1
+        widths, w = [], 4
+        while True:
+            widths.append(w)
+            if w >= pages:
+                break
+            w *= 2
+        for width in widths:
+            for singles in (True, False):
+                key = self._mixed_shape(kernels.bound_rows(tokens), 1, singles, width)
+                if key not in self._graphs:
+                    self._mixed_graph_step([], key)
+                    made += 1
+        return made
 
     def _record(self, key, entries: Sequence[StepEntry]):
         """Records the decode step of size `key` with the entries' rows first and rows of no request

@@ -92,6 +92,9 @@ class LLM:
                 reach = min(reach, max(g.pool.num_pages for g in full) * block_size)
             before = torch.cuda.memory_allocated()
             self.graphs_recorded_at_start = runner.record_decode_graphs(max_batch_size, reach)
+            if chunk_size is not None and max_num_batched_tokens < model.spec.max_positions:
+                # prompts cut into portions under a token budget: the steps of a busy engine hold the budget's tokens
+                self.graphs_recorded_at_start += runner.record_mixed_graphs(max_num_batched_tokens, reach)
             self.graph_memory_bytes = torch.cuda.memory_allocated() - before
             if self.graph_memory_bytes > (4 << 30):
                 import warnings
