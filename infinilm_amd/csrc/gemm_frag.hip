@@ -3,7 +3,7 @@
 //
 // A workgroup of 8 waves takes NT tiles of 16 rows of W and all rows of X.  The waves split the workgroup's
 // range of K evenly; a wave has the W fragments of up to ROUND k-steps in flight at once (a fragment is 1 KB
-// of consecutive bytes: W comes in at the memory's speed) and streams the X fragments of GF_XC steps beside
+// of consecutive bytes: W comes in at the memory's speed) and streams the X fragments of XC steps beside
 // them, a chunk ahead (X is read by every workgroup, from the L2s, also 1 KB an instruction).  The waves'
 // partial tiles meet in LDS and are summed in wave order: the order of a sum depends on K alone, not on the
 // number of rows or on the batch.  The thread that reduces an output applies the epilogue:
@@ -24,7 +24,6 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 #define GF_WAVES 8
-#define GF_XC 2          // k-steps a chunk of X fragments
 #define GF_SS_ROWS 64    // rows of a tile's record of partial sums of squares
 
 enum { GF_PLAIN = 0, GF_SWIGLU = 1, GF_ROPE = 2, GF_TAIL = 3 };
@@ -73,8 +72,12 @@ __global__ void __launch_bounds__(GF_WAVES * 64)
 gemm_frag_kernel(const GfArgs A) {
     __shared__ __align__(16) float part[NT][MG][GF_WAVES][64][4];
     __shared__ __align__(16) float ssr[GF_WAVES][GF_SS_ROWS];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // the wave's number as a scalar: every index of a k-step is then one too, and a load's address a scalar base
+    // plus the lane's offset (as a per-lane value it costs registers for every load, and those run out: the
+    // compiler then parks fragments in scratch memory, which waits for all loads in flight)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int unit = blockIdx.x;
+    constexpr int XC = MG <= 2 ? 4 : 2;   // k-steps a chunk of X fragments (two chunks in flight)
     // ---- the wave's k-steps
     const int p0s = blockIdx.y * A.steps_per_part;
     const int p1s = p0s + A.steps_per_part < A.ksteps ? p0s + A.steps_per_part : A.ksteps;
@@ -117,14 +120,14 @@ gemm_frag_kernel(const GfArgs A) {
 #pragma unroll
             for (int t = 0; t < NT; ++t) a[u][t] = A.Wf[((size_t)(unit * NT + t) * A.ksteps + s) * 64 + lane];
         }
-        uint4 b[2][GF_XC][MG];
+        uint4 b[2][XC][MG];
 #define GF_LOADX(BUF_, U_)                                                                       \
-        _Pragma("unroll") for (int u = 0; u < GF_XC; ++u) {                                      \
+        _Pragma("unroll") for (int u = 0; u < XC; ++u) {                                      \
             const int s = s0 + (U_) + u < s_end ? s0 + (U_) + u : s_end - 1;                     \
             _Pragma("unroll") for (int g = 0; g < MG; ++g) b[BUF_][u][g] = A.Xf[((size_t)s * MG + g) * 64 + lane]; \
         }
 #define GF_MULX(BUF_, U_)                                                                        \
-        _Pragma("unroll") for (int u = 0; u < GF_XC; ++u) {                                      \
+        _Pragma("unroll") for (int u = 0; u < XC; ++u) {                                      \
             const bool ok = s0 + (U_) + u < s_end;                                               \
             _Pragma("unroll") for (int g = 0; g < MG; ++g) {                                     \
                 const uint4 xv = ok ? b[BUF_][u][g] : zero;                                      \
@@ -133,14 +136,14 @@ gemm_frag_kernel(const GfArgs A) {
         }
         GF_LOADX(0, 0)
 #pragma unroll
-        for (int uu = 0; uu < ROUND; uu += 2 * GF_XC) {   // (not `u`: the macros' own loops use that name)
-            if (uu + GF_XC < ROUND) GF_LOADX(1, uu + GF_XC)
+        for (int uu = 0; uu < ROUND; uu += 2 * XC) {   // (not `u`: the macros' own loops use that name)
+            if (uu + XC < ROUND) GF_LOADX(1, uu + XC)
             __builtin_amdgcn_sched_barrier(0);
             GF_MULX(0, uu)
             __builtin_amdgcn_sched_barrier(0);
-            if (uu + 2 * GF_XC < ROUND) GF_LOADX(0, uu + 2 * GF_XC)
+            if (uu + 2 * XC < ROUND) GF_LOADX(0, uu + 2 * XC)
             __builtin_amdgcn_sched_barrier(0);
-            if (uu + GF_XC < ROUND) GF_MULX(1, uu + GF_XC)
+            if (uu + XC < ROUND) GF_MULX(1, uu + XC)
             __builtin_amdgcn_sched_barrier(0);
         }
 #undef GF_LOADX
