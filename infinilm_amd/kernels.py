@@ -319,6 +319,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     # (not for small matrices, whose few tiles leave most of the chip idle whatever the split: 0.5B shape at 128
     # rows 2.22 against 1.96 ms a step with the library)
     if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS and _mid_fills_the_chip(N, K, a.device):
+        # Long chunks of X resident in LDS where a workgroup's range of K is short (the o projection: a range is 2 to 4
+        # chunks, all in flight at once; the kernel that walks K in steps of 64 waits a memory latency a step) or the
+        # rows are many: measured at the 8B shapes, o projection 12.8 against 15.4 us at 72 rows, 14.3 / 17.3 at 96,
+        # 16.7 / 19.4 at 128, 16.5 / 22.2 at 160, 19.5 / 24.8 at 208; down projection 43.8 against 38.3 at 96 and
+        # 48.8 / 41.2 at 128 (stays with the steps of 64), 43.9 / 45.3 at 144, 45.6 / 47.1 at 160, 53.4 / 56.7 at 208
+        if USE_TALL and M <= TALL_MAX_ROWS and (_tall_chunks_per_part(M, N, K) <= 4 or M >= TALL_LONG_K_MIN_ROWS):
+            return _gemm_tall(a, w, K, frag_w)
         return _gemm_mid(a, w, K, False)
     # 17 to 64 rows on their way into the residual sum: K in ranges of 1024 with the X fragments of all rows
     # in registers (o projection at 64 rows 13.1 against the library's 18.9 us, down projection 33.9
@@ -427,6 +434,61 @@ def _gemm_mid(x: torch.Tensor, w: torch.Tensor, K: int, act: bool) -> torch.Tens
     return parts
 
 
+USE_TALL = os.environ.get("INFINILM_AMD_TALL", "1") == "1"
+TALL_MAX_ROWS = 208   # most rows of X of the products that keep long chunks of X in LDS (ilm_gemm_tall_max_rows())
+TALL_TARGET_WGS = int(os.environ.get("INFINILM_AMD_TALL_WGS", "256"))
+TALL_LONG_K_MIN_ROWS = 144     # rows from which a long range of K a workgroup goes to that product too
+TALL_GATEUP_MAX_ROWS = 112     # rows up to which the gate/up projection does (beyond: see gateup_swiglu_gemm)
+
+
+def _tall_chunk(M: int) -> int:
+    """k a chunk of the tall product for M rows (ilm_gemm_tall_chunk())."""
+    return 512 if M <= 64 else (256 if M <= 128 else 128)
+
+
+def _tall_split(M: int, N: int, K: int) -> tuple:
+    """(parts, chunks a part) of the tall product: K split so that the launch has about a workgroup a compute unit."""
+    n_tiles = -(-N // 128)
+    chunks = -(-K // _tall_chunk(M))
+    kb = max(1, min(-(-TALL_TARGET_WGS // n_tiles), chunks))
+    cpp = -(-chunks // kb)
+    return -(-chunks // cpp), cpp
+
+
+def _tall_chunks_per_part(M: int, N: int, K: int) -> int:
+    return _tall_split(M, N, K)[1]
+
+
+def _gemm_tall(x: torch.Tensor, w: torch.Tensor, K: int, frag_w=None) -> torch.Tensor:
+    """17 to 208 rows, result in float32 parts [P, M, N] split over K (see gemm_tall.hip)."""
+    M, N = x.shape[0], w.shape[0]
+    kb, cpp = _tall_split(M, N, K)
+    parts = torch.empty((kb, M, N), dtype=F32, device=x.device)
+    fw = _frag_of(frag_w) if USE_FRAG else None
+    if fw is not None:
+        _run("ilm_gemm_tall", parts.data_ptr(), N, M * N, kb, cpp, fw.data.data_ptr(), 0, M, N, K, x.data_ptr(), x.stride(0), 1,
+             _stream())
+    else:
+        _run("ilm_gemm_tall", parts.data_ptr(), N, M * N, kb, cpp, w.data_ptr(), w.stride(0), M, N, K, x.data_ptr(), x.stride(0),
+             0, _stream())
+    return parts
+
+
+def gemm_tall_swiglu(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], frag_w=None) -> torch.Tensor:
+    """silu(x Wg^T + bg) * (x Wu^T + bu) for 17 to 208 rows, W = [Wg; Wu] (see gemm_tall.hip)."""
+    M, K = x.shape
+    inter = w.shape[0] // 2
+    act = torch.empty((M, inter), dtype=x.dtype, device=x.device)
+    fw = _frag_of(frag_w) if USE_FRAG else None
+    if fw is not None:
+        _run("ilm_gemm_tall_swiglu", act.data_ptr(), act.stride(0), x.data_ptr(), x.stride(0), fw.data.data_ptr(), 0, _ptr(bias),
+             M, inter, K, 1, _stream())
+    else:
+        _run("ilm_gemm_tall_swiglu", act.data_ptr(), act.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
+             _ptr(bias), M, inter, K, 0, _stream())
+    return act
+
+
 USE_GATEUP_SWIGLU = os.environ.get("INFINILM_AMD_GATEUP_SWIGLU", "1") == "1"
 USE_GATEUP_WIDE = os.environ.get("INFINILM_AMD_GATEUP_WIDE", "1") == "1"
 # outputs from which the kernel with X through LDS is used (-1: 48 a compute unit; 0: always, as its tests do)
@@ -502,8 +564,14 @@ def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
     # the library is faster - 2B-family shape, 5,760 outputs, 64 rows: 6.40 against 6.07 ms a step)
     wide_min = GATEUP_WIDE_MIN_OUTPUTS if GATEUP_WIDE_MIN_OUTPUTS >= 0 else 48 * _num_cus(x.device)
     wide = USE_GATEUP_WIDE and not resident and 16 < M <= 64 and w.shape[0] // 2 >= wide_min
+    # 65 to 112 rows, and up to 176 where the rows are no multiple of 32 (the vendor library's product is then slow):
+    # long chunks of X resident in LDS (gemm_tall.hip).  Measured at the 8B shape against the library's product and
+    # the activation kernel: 57.6 against 70.1 us at 72 rows, 61.6 / 66.2 at 96, 66.5 / 81.4 at 112, 71.6 / 69.0 at
+    # 128, 76.1 / 85.2 at 144, 75.4 / 72.7 at 160, 82.8 / 90.1 at 176, 86.6 / 75.6 at 192, 96.6 / 83.0 at 208
+    tall = (USE_TALL and USE_GATEUP_WIDE and row_ss is None and 64 < M <= TALL_MAX_ROWS and w.shape[0] // 2 >= wide_min
+            and (M <= TALL_GATEUP_MAX_ROWS or (M % 32 != 0 and M <= 176)))
     if not (USE_GATEUP_SWIGLU and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and x.is_cuda
-            and (resident or wide) and K % 8 == 0 and w.shape[0] % 2 == 0 and w.shape[1] == K
+            and (resident or wide or tall) and K % 8 == 0 and w.shape[0] % 2 == 0 and w.shape[1] == K
             and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         return None
@@ -511,6 +579,8 @@ def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
     I = w.shape[0] // 2
     if bias is not None and (bias.shape != (2 * I,) or bias.dtype != BF16 or not bias.is_contiguous()):
         raise KernelError("bias does not fit the fused gate/up projection")
+    if tall:
+        return gemm_tall_swiglu(x, w, bias, frag_w)
     out = torch.empty((M, I), dtype=BF16, device=x.device)
     if resident:
         _run("ilm_gemm_gateup_swiglu", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
@@ -604,6 +674,21 @@ def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple
             per_chunk = n
     while per_chunk >= 4 and 2 * per_chunk <= steps and workgroups(2 * per_chunk) >= 2 * cus:
         per_chunk *= 2
+    # More workgroups than the chip holds at once (two a compute unit): they run in rounds, and a last round that is
+    # nearly empty costs as much as a full one.  Among chunks of a quarter to twice that length take the one with the
+    # least rounds x (steps a chunk + a workgroup's fixed cost, about three quarters of a step) + the chunks' merge.
+    # Measured at the 8B head shape, 4096 keys, kernel + merge: 80 tokens 80.7 us with 512 keys a chunk (1024: 91.1),
+    # 96 tokens 89.1 with 512 (1024: 95.9), 160 tokens 148.4 with 512 (2048: 170.4), 192 tokens 159.0 with 1024
+    # (2048: 174.9); 160 tokens over 8192 keys 267.4 with 1024 (4096: 317.7).
+    slots = 2 * cus
+    if workgroups(per_chunk) > slots:
+        def cost(n):
+            return -(-workgroups(n) // slots) * (0.75 + n) + 0.15 * -(-steps // n)
+        best = per_chunk
+        for n in (per_chunk * 2, per_chunk // 2, per_chunk // 4):
+            if 2 <= n <= steps and (cost(n), -n) < (cost(best), -best):
+                best = n
+        per_chunk = best
     while -(-steps // per_chunk) > ATT_MAX_CHUNKS:
         per_chunk += 1
     span = per_chunk * ATT_STEP

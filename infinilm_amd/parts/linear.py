@@ -52,7 +52,7 @@ class FusedLinear:
                 allow_parts: bool = False) -> torch.Tensor:
         """`allow_parts`: the result may come as float32 parts [P, T, out] still to be summed; only for a
         result that goes straight into `ResidualStream.push` (the next norm's kernel sums them)."""
-        frag = self.frag_weight if kernels.frag_weight_ok(self.weight) and x.shape[0] <= kernels.FRAG_MAX_ROWS else None
+        frag = self.frag_weight if kernels.frag_weight_ok(self.weight) and x.shape[0] <= max(kernels.FRAG_MAX_ROWS, kernels.TALL_MAX_ROWS) else None
         return kernels.gemm(x, self.weight, self.bias, alpha, out_dtype, allow_parts=allow_parts, frag_w=frag)
 
 

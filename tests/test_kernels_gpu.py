@@ -299,8 +299,64 @@ def test_gate_up_projection_with_the_activation_in_its_epilogue(K, monkeypatch, 
     assert (act.float() - two.float()).abs().max() <= 2 ** -6 * max(float(two.float().abs().max()), 1e-6)
     assert K.gateup_swiglu_gemm(dev(x.float()), dev(w.float()), None) is None          # float32: not this kernel
     if M <= 32:
-        big = _rand((65, Kd), 34, torch.bfloat16)
+        big = _rand((209, Kd), 34, torch.bfloat16)
         assert K.gateup_swiglu_gemm(dev(big), dev(w), dev(b)) is None                  # too many rows
+
+
+@pytest.mark.parametrize("M,N,K_", [(17, 200, 264), (64, 128, 1024), (65, 334, 520), (100, 4096, 4096), (128, 130, 16384),
+                                    (129, 256, 640), (144, 4096, 16384), (208, 512, 2048), (97, 64, 72), (113, 1030, 4104)])
+def test_products_with_long_chunks_of_x_in_lds(K, monkeypatch, M, N, K_):
+    """`gemm_tall.hip`, both epilogues, weights in plain rows and in fragment order, against the plain formulas:
+    chunks of 512, 256 and 128 k (by the rows of X), K no multiple of a chunk, rows and outputs no multiple of a
+    tile, one part and many; and where the engine's path takes it."""
+    from infinilm_amd.csrc import lib
+    assert K.TALL_MAX_ROWS == lib.load().ilm_gemm_tall_max_rows()
+    assert all(K._tall_chunk(m) == lib.load().ilm_gemm_tall_chunk(m) for m in (17, 64, 65, 128, 129, 208))
+    x, w = _rand((M, K_), 41, torch.bfloat16), _rand((N, K_), 42, torch.bfloat16, 0.05)
+    want = P.plain_linear(x.to(F64), w.to(F64))
+    for fw in (None, K.pack_weight(w.to(DEV))):
+        parts = K._gemm_tall(x.to(DEV), w.to(DEV), K_, fw)
+        assert parts.dtype == torch.float32 and parts.shape == (K._tall_split(M, N, K_)[0], M, N)
+        _close(parts.sum(0), want, 1e-5)
+    if M > 64 and K._mid_fills_the_chip(N, K_, torch.device(DEV)):
+        took = []
+        monkeypatch.setattr(K, "_gemm_tall", lambda *a, **k: took.append("tall") or torch.zeros(1, M, N, device=DEV))
+        monkeypatch.setattr(K, "_gemm_mid", lambda *a, **k: took.append("mid") or torch.zeros(1, M, N, device=DEV))
+        K.gemm(x.to(DEV), w.to(DEV), allow_parts=True)
+        assert took == ["tall" if K._tall_chunks_per_part(M, N, K_) <= 4 or M >= K.TALL_LONG_K_MIN_ROWS else "mid"]
+        monkeypatch.undo()
+    inter = N // 2
+    bias = _rand((2 * inter,), 43, torch.bfloat16, 0.1)
+    wg = w[:2 * inter]
+    y = P.plain_linear(x.to(F64), wg.to(F64), bias.to(F64))
+    want_act = P.plain_swiglu(y[:, :inter], y[:, inter:])
+    two = K.swiglu(K.gemm(x.to(DEV), wg.to(DEV), bias.to(DEV)))
+    for fw in (None, K.pack_weight(wg.to(DEV), "gate_up8")):
+        for b in (bias.to(DEV), None):
+            act = K.gemm_tall_swiglu(x.to(DEV), wg.to(DEV), b, fw)
+            assert act.shape == (M, inter) and act.dtype == torch.bfloat16
+            if b is None:
+                y0 = P.plain_linear(x.to(F64), wg.to(F64))
+                _close(act, P.plain_swiglu(y0[:, :inter], y0[:, inter:]), 1e-2)
+            else:
+                _close(act, want_act, 1e-2)
+                # gate and up are rounded to bfloat16 at the same place as the projection followed by the activation kernel
+                assert (act.float() - two.float()).abs().max() <= 2 ** -6 * max(float(two.float().abs().max()), 1e-6)
+
+
+def test_where_the_gate_up_projection_keeps_x_in_lds(K, monkeypatch):
+    """65 to 112 rows, and up to 176 rows that are no multiple of 32, take the kernel with long chunks of X in LDS
+    when the outputs fill the chip; other row counts are left to the library's product and the activation kernel."""
+    monkeypatch.setattr(K, "GATEUP_WIDE_MIN_OUTPUTS", 0)
+    w = _rand((2 * 96, 72), 44, torch.bfloat16, 0.1).to(DEV)
+    for M, taken in ((65, True), (96, True), (112, True), (113, True), (128, False), (144, True), (160, False), (176, True), (192, False),
+                     (175, True), (177, False), (208, False), (209, False)):
+        x = _rand((M, 72), 45, torch.bfloat16).to(DEV)
+        act = K.gateup_swiglu_gemm(x, w, None)
+        assert (act is not None) == taken, M
+        if taken:
+            y = P.plain_linear(x.to(F64), w.to(F64))
+            _close(act, P.plain_swiglu(y[:, :96], y[:, 96:]), 1e-2)
 
 
 @pytest.mark.parametrize("M,Ko,H,I,bias,wdt", [(8, 4096, 4096, 16384, False, torch.bfloat16), (3, 96, 80, 200, True, torch.float32),
