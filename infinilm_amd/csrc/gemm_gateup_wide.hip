@@ -62,7 +62,11 @@ gemm_gateup_wide_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const 
     // Loads are unconditional 16-byte loads from clamped addresses; what lies beyond K or beyond M is
     // replaced by zeros on the X side, which makes the clamped W loads harmless.  The X pieces are plain
     // variables: a register array indexed inside a macro's loop lands in scratch memory, and every
-    // access to that waits for all loads in flight.
+    // access to that waits for all loads in flight.  A piece is looked at only when it is stored into LDS (a
+    // select right after its load would make the wave wait for it there), and the next step's loads are issued
+    // without a branch around them (after the last step: that step's again, for nothing): behind a branch the
+    // compiler cannot count how many loads are younger than the fragments it is about to use, and waits for the
+    // new ones.
 #define GW_LOAD_W(DST_, STEP_)                                                   \
     _Pragma("unroll") for (int s = 0; s < GW_KSUB; ++s) {                        \
         if (FRAGW) {                                                             \
@@ -76,20 +80,24 @@ gemm_gateup_wide_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const 
 #define GW_X1(XV_, I_)                                                           \
     if (XPER > I_) {                                                             \
         const int row = xr + RPP * I_;                                           \
-        const uint4 v = *reinterpret_cast<const uint4*>(X + (size_t)(row < M ? row : 0) * lda + (size_t)k8c * 8); \
-        XV_ = (row < M && kin) ? v : zero;                                       \
+        XV_ = *reinterpret_cast<const uint4*>(X + (size_t)(row < M ? row : 0) * lda + (size_t)k8c * 8); \
     }
 #define GW_LOAD_X(STEP_)                                                         \
     {                                                                            \
         const int k8 = (STEP_) * PR + xk;                                        \
-        const bool kin = k8 <= k8_last;                                          \
-        const int k8c = kin ? k8 : k8_last;                                      \
+        const int k8c = k8 <= k8_last ? k8 : k8_last;                            \
         GW_X1(x0, 0) GW_X1(x1, 1) GW_X1(x2, 2) GW_X1(x3, 3) GW_X1(x4, 4) GW_X1(x5, 5) GW_X1(x6, 6) GW_X1(x7, 7) \
     }
-#define GW_S1(XV_, I_, B_) \
-    if (XPER > I_) *reinterpret_cast<uint4*>(xs + (B_) * XBUF + RPP * I_ * XROW) = XV_;
-#define GW_STORE_X(BUF_)                                                         \
-    { GW_S1(x0, 0, BUF_) GW_S1(x1, 1, BUF_) GW_S1(x2, 2, BUF_) GW_S1(x3, 3, BUF_) GW_S1(x4, 4, BUF_) GW_S1(x5, 5, BUF_) GW_S1(x6, 6, BUF_) GW_S1(x7, 7, BUF_) }
+#define GW_S1(XV_, I_, B_)                                                                           \
+    if (XPER > I_) {                                                                                 \
+        const unsigned mk = (kin && xr + RPP * I_ < M) ? 0xffffffffu : 0u;   /* (a select between two 16-byte structs goes through memory) */ \
+        *reinterpret_cast<uint4*>(xs + (B_) * XBUF + RPP * I_ * XROW) = make_uint4(XV_.x & mk, XV_.y & mk, XV_.z & mk, XV_.w & mk); \
+    }
+#define GW_STORE_X(BUF_, STEP_)                                                  \
+    {                                                                            \
+        const bool kin = (STEP_) * PR + xk <= k8_last;                           \
+        GW_S1(x0, 0, BUF_) GW_S1(x1, 1, BUF_) GW_S1(x2, 2, BUF_) GW_S1(x3, 3, BUF_) GW_S1(x4, 4, BUF_) GW_S1(x5, 5, BUF_) GW_S1(x6, 6, BUF_) GW_S1(x7, 7, BUF_) \
+    }
 
     f32x4 acc[MG];
 #pragma unroll
@@ -101,7 +109,7 @@ gemm_gateup_wide_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const 
 #pragma unroll
     for (int j = 0; j < GW_AHEAD; ++j)
         if (j < nsteps) GW_LOAD_W(w[j], j)
-    GW_STORE_X(0)
+    GW_STORE_X(0, 0)
     __syncthreads();
     for (int base = 0; base < nsteps; base += GW_AHEAD + 1) {
 #pragma unroll
@@ -111,8 +119,12 @@ gemm_gateup_wide_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const 
                 const int buf = step & 1;
                 // X of the next step first: the wait for it before the store below then leaves the W loads,
                 // issued later and coming from memory, in flight
-                if (step + 1 < nsteps) GW_LOAD_X(step + 1)
-                if (step + GW_AHEAD < nsteps) GW_LOAD_W(w[(j + GW_AHEAD) % (GW_AHEAD + 1)], step + GW_AHEAD)
+                {
+                    const int nx = step + 1 < nsteps ? step + 1 : nsteps - 1;
+                    const int nw = step + GW_AHEAD < nsteps ? step + GW_AHEAD : nsteps - 1;
+                    GW_LOAD_X(nx)
+                    GW_LOAD_W(w[(j + GW_AHEAD) % (GW_AHEAD + 1)], nw)
+                }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int s = 0; s < GW_KSUB; ++s) {
@@ -124,7 +136,9 @@ gemm_gateup_wide_kernel(bf16* __restrict__ C, const bf16* __restrict__ X, const 
                     for (int g = 0; g < MG; ++g) acc[g] = gw_mfma(w[j][s], b[g], acc[g]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (step + 1 < nsteps) GW_STORE_X(buf ^ 1)   // its readers passed the barrier one step ago
+                // (its readers passed the barrier one step ago; after the last step the stored tile is not read: the
+                // store is unconditional so that the compiler does not move the loads down into a branch beside it)
+                GW_STORE_X(buf ^ 1, step + 1 < nsteps ? step + 1 : nsteps - 1)
                 __syncthreads();
             }
         }
