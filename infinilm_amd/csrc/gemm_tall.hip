@@ -2,12 +2,14 @@
 // projections of a decode step with many requests, or of a small portion of a prompt.
 //
 // A workgroup of 8 waves takes 128 rows of W (a tile of 16 a wave) and all rows of X, and walks its range of K in
-// chunks of KC (512 up to 64 rows of X, 256 up to 128, 128 beyond: two chunks of X fill most of a compute unit's
-// 160 KB of LDS).  A chunk of X goes from plain rows into LDS in fragment order: whole 128-byte lines of 8 rows
-// an instruction on the memory side, and on the LDS side the 1 KB that one matrix operand reads lies in the
-// lanes' order, so neither padding nor exchange of pieces is needed for reads without bank conflicts.  The next
-// chunk's X (in registers) and W fragments are on their way while this one is multiplied: one barrier a chunk,
-// a quarter to an eighth of what steps of 64 k need, and 128 KB a compute unit in flight.  A wave streams its
+// chunks of KC = 64 or 128 k, two of which lie in LDS.  A chunk of X goes from plain rows into LDS in fragment
+// order: whole 128-byte lines of 8 rows an instruction on the memory side, and on the LDS side the 1 KB that one
+// matrix operand reads lies in the lanes' order, so neither padding nor exchange of pieces is needed for reads
+// without bank conflicts.  The next chunk's X (in registers) and W fragments are on their way while this one is
+// multiplied, one barrier a chunk.  Up to 128 rows of X a workgroup stays within 128 registers and 64 KB of LDS,
+// so that two share a compute unit and one's barrier and waits are covered by the other (measured at the 8B
+// shapes: chunks of 256 and 512 k, which fill the unit's 160 KB of LDS with one workgroup, were slower at every
+// row count: gate/up at 64 rows 56.2 and 58.3 us against 53.2 with chunks of 128).  A wave streams its
 // own W rows straight into v_mfma_f32_16x16x32_bf16 fragments (from plain rows, or 1 KB of consecutive bytes a
 // fragment where the weight is given in fragment order, frag.h); no reduction between waves.
 //
@@ -47,14 +49,15 @@ __device__ __forceinline__ f32x4 gt_mfma(uint4 a, uint4 b, f32x4 c) {
 // MG: groups of 16 rows of X; KC: k a chunk; FRAGW: W in fragment order (parts: tiles of 16 consecutive rows; swiglu:
 // tiles of 8 gate + 8 up rows)
 template <int MG, int KC, bool FRAGW, int EPI>
-__global__ void __launch_bounds__(GT_THREADS)
+__global__ void __launch_bounds__(GT_THREADS, MG <= 8 ? 4 : 2)
 gemm_tall_kernel(const GtArgs A) {
     constexpr int KS = KC / 32;                 // matrix-core k-steps a chunk
     constexpr int LINES = KC / 64;              // 128-byte lines a row of a chunk
     constexpr int BLOCKS = MG * 2 * LINES;      // staging blocks (8 rows x one line) a chunk
     constexpr int XPER = (BLOCKS + GT_WAVES - 1) / GT_WAVES;
     static_assert(XPER <= 8, "a chunk of X is at most eight 16-byte pieces a thread");
-    static_assert(2 * KS * MG <= 144, "two chunks of X fit the LDS of a compute unit");
+    static_assert(KC == 64 || KC == 128, "chunks of 64 or 128 k");
+    static_assert(2 * KS * MG <= (MG <= 8 ? 64 : 144), "two chunks of X fit the LDS (of half a compute unit up to 128 rows)");
     __shared__ __align__(16) uint4 Xs[2][KS][MG][64];
     // the wave's number as a scalar: what depends on it stays in scalar registers
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -239,73 +242,70 @@ gemm_tall_kernel(const GtArgs A) {
 
 extern "C" int ilm_gemm_tall_max_rows() { return 208; }
 
-// k a chunk for M rows of X (what two chunks of X in LDS allow)
-static int gt_chunk(int M) { return M <= 64 ? 512 : (M <= 128 ? 256 : 128); }
-extern "C" int ilm_gemm_tall_chunk(int M) { return gt_chunk(M); }
-
 template <int EPI>
-static void gt_launch(const GtArgs& a, dim3 grid, int frag_w, hipStream_t stream) {
+static void gt_launch(const GtArgs& a, int kc, dim3 grid, int frag_w, hipStream_t stream) {
 #define GT_GO(MG_, KC_)                                                                                        \
     if (frag_w) gemm_tall_kernel<MG_, KC_, true, EPI><<<grid, GT_THREADS, 0, stream>>>(a);                     \
     else gemm_tall_kernel<MG_, KC_, false, EPI><<<grid, GT_THREADS, 0, stream>>>(a)
+#define GT_KC(MG_) if (kc == 64) { GT_GO(MG_, 64); } else { GT_GO(MG_, 128); }
     switch ((a.M + 15) / 16) {
-        case 2: GT_GO(2, 512); break;
-        case 3: GT_GO(3, 512); break;
-        case 4: GT_GO(4, 512); break;
-        case 5: GT_GO(5, 256); break;
-        case 6: GT_GO(6, 256); break;
-        case 7: GT_GO(7, 256); break;
-        case 8: GT_GO(8, 256); break;
-        case 9: GT_GO(9, 128); break;
-        case 10: GT_GO(10, 128); break;
-        case 11: GT_GO(11, 128); break;
-        case 12: GT_GO(12, 128); break;
-        default: GT_GO(13, 128); break;
+        case 2: GT_KC(2) break;
+        case 3: GT_KC(3) break;
+        case 4: GT_KC(4) break;
+        case 5: GT_KC(5) break;
+        case 6: GT_KC(6) break;
+        case 7: GT_KC(7) break;
+        case 8: GT_KC(8) break;
+        case 9: GT_KC(9) break;
+        case 10: GT_KC(10) break;
+        case 11: GT_KC(11) break;
+        case 12: GT_KC(12) break;
+        default: GT_KC(13) break;
     }
+#undef GT_KC
 #undef GT_GO
 }
 
-static int gt_check(const char* what, int M, int N, int K, const void* X, int lda, const void* W, int ldw, int frag_w) {
+static int gt_check(const char* what, int M, int N, int K, int kc, const void* X, int lda, const void* W, int ldw, int frag_w) {
     ILM_REQUIRE(M > 16 && M <= 208 && N > 0 && K > 0, "%s: needs 17 <= M <= 208, got M=%d N=%d K=%d", what, M, N, K);
+    ILM_REQUIRE(kc == 64 || kc == 128, "%s: chunks of %d k (64 or 128)", what, kc);
     ILM_REQUIRE(K % 8 == 0 && lda % 8 == 0 && lda >= K && (frag_w || (ldw % 8 == 0 && ldw >= K)), "%s: K=%d lda=%d ldw=%d", what,
                 K, lda, ldw);
     ILM_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "%s: operands must be 16-byte aligned", what);
     return 0;
 }
 
-// C: float [kb][M][ldc] with c_part_stride elements between the parts; part y covers chunks_per_part chunks of
-// ilm_gemm_tall_chunk(M) k from y * chunks_per_part on, kb = ceil(ceil(K / chunk) / chunks_per_part).
+// C: float [kb][M][ldc] with c_part_stride elements between the parts; part y covers chunks_per_part chunks of kc k
+// (64 or 128) from y * chunks_per_part on, kb = ceil(ceil(K / kc) / chunks_per_part).
 // frag_w != 0: W is the weight in fragment order, tiles of 16 consecutive rows (ldw is not used).
-extern "C" int ilm_gemm_tall(void* C, int ldc, long c_part_stride, int kb, int chunks_per_part, const void* W, int ldw, int M,
-                             int N, int K, const void* X, int lda, int frag_w, hipStream_t stream) {
-    if (gt_check("gemm_tall", M, N, K, X, lda, W, ldw, frag_w)) return -1;
+extern "C" int ilm_gemm_tall(void* C, int ldc, long c_part_stride, int kb, int chunks_per_part, int kc, const void* W, int ldw,
+                             int M, int N, int K, const void* X, int lda, int frag_w, hipStream_t stream) {
+    if (gt_check("gemm_tall", M, N, K, kc, X, lda, W, ldw, frag_w)) return -1;
     GtArgs a = {};
     a.X = (const bf16*)X; a.W = (const bf16*)W; a.M = M; a.N = N; a.K = K; a.lda = lda; a.ldw = ldw;
-    const int kc = gt_chunk(M);
     a.chunks = (K + kc - 1) / kc;
     a.chunks_per_part = chunks_per_part;
     ILM_REQUIRE(chunks_per_part > 0 && kb == (a.chunks + chunks_per_part - 1) / chunks_per_part && kb <= 65535,
                 "gemm_tall: %d parts of %d chunks do not cover the %d chunks of K=%d", kb, chunks_per_part, a.chunks, K);
     ILM_REQUIRE(ldc >= N && ((uintptr_t)C & 15) == 0, "gemm_tall: ldc=%d", ldc);
     a.C = (float*)C; a.ldc = ldc; a.part_stride = (size_t)c_part_stride;
-    gt_launch<GT_PARTS>(a, dim3((N + GT_NT - 1) / GT_NT, kb), frag_w, stream);
+    gt_launch<GT_PARTS>(a, kc, dim3((N + GT_NT - 1) / GT_NT, kb), frag_w, stream);
     ILM_LAUNCH_CHECK("gemm_tall");
     return 0;
 }
 
-// act [M, ld_act] = silu(X Wg^T + bg) * (X Wu^T + bu) with W = [Wg; Wu] of 2 I rows (bias of 2 I entries or null).
-// frag_w != 0: W is the weight in fragment order with tiles of 8 gate + 8 up rows (ldw is not used).
+// act [M, ld_act] = silu(X Wg^T + bg) * (X Wu^T + bu) with W = [Wg; Wu] of 2 I rows (bias of 2 I entries or null); kc: k a
+// chunk (64 or 128).  frag_w != 0: W is the weight in fragment order with tiles of 8 gate + 8 up rows (ldw is not used).
 extern "C" int ilm_gemm_tall_swiglu(void* act, int ld_act, const void* X, int lda, const void* W, int ldw, const void* bias,
-                                    int M, int I, int K, int frag_w, hipStream_t stream) {
-    if (gt_check("gemm_tall_swiglu", M, I, K, X, lda, W, ldw, frag_w)) return -1;
+                                    int M, int I, int K, int kc, int frag_w, hipStream_t stream) {
+    if (gt_check("gemm_tall_swiglu", M, I, K, kc, X, lda, W, ldw, frag_w)) return -1;
     ILM_REQUIRE(ld_act >= I, "gemm_tall_swiglu: ld_act=%d", ld_act);
     GtArgs a = {};
     a.X = (const bf16*)X; a.W = (const bf16*)W; a.bias = (const bf16*)bias; a.M = M; a.N = I; a.K = K; a.lda = lda; a.ldw = ldw;
-    const int kc = gt_chunk(M);
     a.chunks = (K + kc - 1) / kc;
     a.chunks_per_part = a.chunks;
     a.act = (bf16*)act; a.ld_act = ld_act;
-    gt_launch<GT_SWIGLU>(a, dim3((I + GT_NT / 2 - 1) / (GT_NT / 2), 1), frag_w, stream);
+    gt_launch<GT_SWIGLU>(a, kc, dim3((I + GT_NT / 2 - 1) / (GT_NT / 2), 1), frag_w, stream);
     ILM_LAUNCH_CHECK("gemm_tall_swiglu");
     return 0;
 }

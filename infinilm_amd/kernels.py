@@ -318,14 +318,15 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     # at 160, 114 -> 48 at 192, 63 -> 51 at 208; o projection 22 -> 17, 25 -> 19, 32 -> 23 at 192)
     # (not for small matrices, whose few tiles leave most of the chip idle whatever the split: 0.5B shape at 128
     # rows 2.22 against 1.96 ms a step with the library)
+    # 17 to 208 rows on their way into the residual sum: chunks of X resident in LDS, two workgroups a compute unit
+    # (gemm_tall.hip).  Measured at the 8B shapes against the kernels it took over from: o projection 9.8 us against
+    # 10.6 (K ranges of 1024, X in registers) at 32 rows, 11.0 / 12.4 at 64, 12.8 / 17.1 (steps of 64 k, X through LDS)
+    # at 96, 15.8 / 19.4 at 128, 16.9 / 22.2 at 160; down projection 27.7 / 33.1 (four parts of 4096, X in registers) at
+    # 32 rows, 30.3 / 33.3 at 64, 33.7 / 38.1 at 96, 37.1 / 42.0 at 128, 46.2 / 47.1 at 160, 52.0 / 56.7 at 208
+    if (fast and aligned and plain and allow_parts and out is None and USE_TALL and TALL_MIN_ROWS <= M <= TALL_MAX_ROWS
+            and M > 16 and _mid_fills_the_chip(N, K, a.device)):
+        return _gemm_tall(a, w, K, frag_w)
     if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS and _mid_fills_the_chip(N, K, a.device):
-        # Long chunks of X resident in LDS where a workgroup's range of K is short (the o projection: a range is 2 to 4
-        # chunks, all in flight at once; the kernel that walks K in steps of 64 waits a memory latency a step) or the
-        # rows are many: measured at the 8B shapes, o projection 12.8 against 15.4 us at 72 rows, 14.3 / 17.3 at 96,
-        # 16.7 / 19.4 at 128, 16.5 / 22.2 at 160, 19.5 / 24.8 at 208; down projection 43.8 against 38.3 at 96 and
-        # 48.8 / 41.2 at 128 (stays with the steps of 64), 43.9 / 45.3 at 144, 45.6 / 47.1 at 160, 53.4 / 56.7 at 208
-        if USE_TALL and M <= TALL_MAX_ROWS and (_tall_chunks_per_part(M, N, K) <= 4 or M >= TALL_LONG_K_MIN_ROWS):
-            return _gemm_tall(a, w, K, frag_w)
         return _gemm_mid(a, w, K, False)
     # 17 to 64 rows on their way into the residual sum: K in ranges of 1024 with the X fragments of all rows
     # in registers (o projection at 64 rows 13.1 against the library's 18.9 us, down projection 33.9
@@ -435,46 +436,48 @@ def _gemm_mid(x: torch.Tensor, w: torch.Tensor, K: int, act: bool) -> torch.Tens
 
 
 USE_TALL = os.environ.get("INFINILM_AMD_TALL", "1") == "1"
-TALL_MAX_ROWS = 208   # most rows of X of the products that keep long chunks of X in LDS (ilm_gemm_tall_max_rows())
-TALL_TARGET_WGS = int(os.environ.get("INFINILM_AMD_TALL_WGS", "256"))
-TALL_LONG_K_MIN_ROWS = 144     # rows from which a long range of K a workgroup goes to that product too
-TALL_GATEUP_MAX_ROWS = 112     # rows up to which the gate/up projection does (beyond: see gateup_swiglu_gemm)
+TALL_MIN_ROWS = int(os.environ.get("INFINILM_AMD_TALL_MIN_ROWS", "17"))
+TALL_MAX_ROWS = 208   # most rows of X of the products that keep chunks of X in LDS (ilm_gemm_tall_max_rows())
+TALL_MAX_PARTS = 16
+TALL_GATEUP_MAX_ROWS = 112     # rows up to which the gate/up projection takes that product (beyond: see gateup_swiglu_gemm)
 
 
-def _tall_chunk(M: int) -> int:
-    """k a chunk of the tall product for M rows (ilm_gemm_tall_chunk())."""
-    return 512 if M <= 64 else (256 if M <= 128 else 128)
-
-
-def _tall_split(M: int, N: int, K: int) -> tuple:
-    """(parts, chunks a part) of the tall product: K split so that the launch has about a workgroup a compute unit."""
+def _tall_plan(M: int, N: int, K: int) -> tuple:
+    """(k a chunk, parts, chunks a part) of the tall product with parts: chunks of 128 k and K split so that the launch
+    has about a workgroup a compute unit; where a part would then be longer than 1024 k (the down projection), chunks
+    of 64 k and two workgroups a unit, up to 128 rows.  Measured at the 8B shapes, down projection: 30.3 us with
+    chunks of 64 and 512 workgroups against 32.2 with chunks of 128 and 256 at 64 rows, 33.7 / 35.0 at 96, 37.1 / 42.3
+    at 128, 60.7 / 52.0 at 208 (and the step at 160 rows 11.17 against 11.00 ms); o projection 12.5 / 11.0 at 64 rows,
+    14.6 / 12.8 at 96."""
     n_tiles = -(-N // 128)
-    chunks = -(-K // _tall_chunk(M))
-    kb = max(1, min(-(-TALL_TARGET_WGS // n_tiles), chunks))
-    cpp = -(-chunks // kb)
-    return -(-chunks // cpp), cpp
+
+    def split(kc, wgs):
+        chunks = -(-K // kc)
+        kb = max(1, min(-(-wgs // n_tiles), chunks, TALL_MAX_PARTS))
+        cpp = -(-chunks // kb)
+        return kc, -(-chunks // cpp), cpp
+    plan = split(128, 256)
+    if plan[2] > 8 and M <= 128:
+        plan = split(64, 512)
+    return plan
 
 
-def _tall_chunks_per_part(M: int, N: int, K: int) -> int:
-    return _tall_split(M, N, K)[1]
-
-
-def _gemm_tall(x: torch.Tensor, w: torch.Tensor, K: int, frag_w=None) -> torch.Tensor:
+def _gemm_tall(x: torch.Tensor, w: torch.Tensor, K: int, frag_w=None, plan: Optional[tuple] = None) -> torch.Tensor:
     """17 to 208 rows, result in float32 parts [P, M, N] split over K (see gemm_tall.hip)."""
     M, N = x.shape[0], w.shape[0]
-    kb, cpp = _tall_split(M, N, K)
+    kc, kb, cpp = plan or _tall_plan(M, N, K)
     parts = torch.empty((kb, M, N), dtype=F32, device=x.device)
     fw = _frag_of(frag_w) if USE_FRAG else None
     if fw is not None:
-        _run("ilm_gemm_tall", parts.data_ptr(), N, M * N, kb, cpp, fw.data.data_ptr(), 0, M, N, K, x.data_ptr(), x.stride(0), 1,
-             _stream())
+        _run("ilm_gemm_tall", parts.data_ptr(), N, M * N, kb, cpp, kc, fw.data.data_ptr(), 0, M, N, K, x.data_ptr(), x.stride(0),
+             1, _stream())
     else:
-        _run("ilm_gemm_tall", parts.data_ptr(), N, M * N, kb, cpp, w.data_ptr(), w.stride(0), M, N, K, x.data_ptr(), x.stride(0),
-             0, _stream())
+        _run("ilm_gemm_tall", parts.data_ptr(), N, M * N, kb, cpp, kc, w.data_ptr(), w.stride(0), M, N, K, x.data_ptr(),
+             x.stride(0), 0, _stream())
     return parts
 
 
-def gemm_tall_swiglu(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], frag_w=None) -> torch.Tensor:
+def gemm_tall_swiglu(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], frag_w=None, kc: int = 128) -> torch.Tensor:
     """silu(x Wg^T + bg) * (x Wu^T + bu) for 17 to 208 rows, W = [Wg; Wu] (see gemm_tall.hip)."""
     M, K = x.shape
     inter = w.shape[0] // 2
@@ -482,10 +485,10 @@ def gemm_tall_swiglu(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
     fw = _frag_of(frag_w) if USE_FRAG else None
     if fw is not None:
         _run("ilm_gemm_tall_swiglu", act.data_ptr(), act.stride(0), x.data_ptr(), x.stride(0), fw.data.data_ptr(), 0, _ptr(bias),
-             M, inter, K, 1, _stream())
+             M, inter, K, kc, 1, _stream())
     else:
         _run("ilm_gemm_tall_swiglu", act.data_ptr(), act.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
-             _ptr(bias), M, inter, K, 0, _stream())
+             _ptr(bias), M, inter, K, kc, 0, _stream())
     return act
 
 
@@ -564,12 +567,13 @@ def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
     # the library is faster - 2B-family shape, 5,760 outputs, 64 rows: 6.40 against 6.07 ms a step)
     wide_min = GATEUP_WIDE_MIN_OUTPUTS if GATEUP_WIDE_MIN_OUTPUTS >= 0 else 48 * _num_cus(x.device)
     wide = USE_GATEUP_WIDE and not resident and 16 < M <= 64 and w.shape[0] // 2 >= wide_min
-    # 65 to 112 rows, and up to 176 where the rows are no multiple of 32 (the vendor library's product is then slow):
-    # long chunks of X resident in LDS (gemm_tall.hip).  Measured at the 8B shape against the library's product and
-    # the activation kernel: 57.6 against 70.1 us at 72 rows, 61.6 / 66.2 at 96, 66.5 / 81.4 at 112, 71.6 / 69.0 at
-    # 128, 76.1 / 85.2 at 144, 75.4 / 72.7 at 160, 82.8 / 90.1 at 176, 86.6 / 75.6 at 192, 96.6 / 83.0 at 208
-    tall = (USE_TALL and USE_GATEUP_WIDE and row_ss is None and 64 < M <= TALL_MAX_ROWS and w.shape[0] // 2 >= wide_min
-            and (M <= TALL_GATEUP_MAX_ROWS or (M % 32 != 0 and M <= 176)))
+    # 17 to 112 rows, and up to 176 where the rows are no multiple of 32 (the vendor library's product is then slow):
+    # chunks of X resident in LDS, two workgroups a compute unit (gemm_tall.hip).  Measured at the 8B shape: 48.1 us
+    # against 52.9 (X in registers, two row groups) at 32 rows, 53.2 against 57.4 (X through LDS in steps of 256 k, one
+    # workgroup a unit) at 64; against the library's product and the activation kernel 57.7 / 66.2 at 96, 66.5 / 81.4 at
+    # 112, 71.2 / 69.0 at 128, 76.1 / 85.2 at 144, 75.3 / 72.7 at 160, 82.8 / 90.1 at 176, 86.6 / 75.6 at 192, 90.4 / 83.0 at 208
+    tall = (USE_TALL and USE_GATEUP_WIDE and row_ss is None and max(TALL_MIN_ROWS, 17) <= M <= TALL_MAX_ROWS
+            and w.shape[0] // 2 >= wide_min and (M <= TALL_GATEUP_MAX_ROWS or (M % 32 != 0 and M <= 176)))
     if not (USE_GATEUP_SWIGLU and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and x.is_cuda
             and (resident or wide or tall) and K % 8 == 0 and w.shape[0] % 2 == 0 and w.shape[1] == K
             and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0

@@ -221,8 +221,12 @@ def test_gemm_bfloat16(K, M, N, K_, out_dtype):
                                     (48, 331, 200), (35, 50, 8200), (128, 1030, 1096), (97, 64, 72), (32, 4096, 16384),
                                     (20, 331, 12296), (27, 50, 8200), (5, 96, 5760), (30, 2304, 5760), (192, 4096, 16384), (208, 331, 4096),
                                     (150, 331, 1096), (177, 96, 200)])
-def test_gemm_split_over_k_and_its_consumer(K, monkeypatch, M, N, K_):
-    """Few rows and long K: the product comes as float32 parts; add_rmsnorm sums them in order."""
+@pytest.mark.parametrize("tall", [True, False])
+def test_gemm_split_over_k_and_its_consumer(K, monkeypatch, M, N, K_, tall):
+    """Few rows and long K: the product comes as float32 parts; add_rmsnorm sums them in order.  `tall`: with the
+    product that keeps chunks of X in LDS (17 to 208 rows of a matrix that fills the chip), and with the kernels
+    that serve when it is switched off."""
+    monkeypatch.setattr(K, "USE_TALL", tall)
     a, w = _rand((M, K_), 14, torch.bfloat16), _rand((N, K_), 15, torch.bfloat16, 0.05)
     small = M > 64 and not K._mid_fills_the_chip(N, K_, torch.device(DEV))
     if small:
@@ -230,7 +234,9 @@ def test_gemm_split_over_k_and_its_consumer(K, monkeypatch, M, N, K_):
         assert K.gemm(a.to(DEV), w.to(DEV), allow_parts=True).dtype == torch.bfloat16
         monkeypatch.setattr(K, "MID_MIN_WGS_PER_CU", -1.0)
     parts = K.gemm(a.to(DEV), w.to(DEV), allow_parts=True)
-    if 16 < M <= 64 and K_ % 8 == 0:   # K ranges of 1024 (up to 32 rows with K beyond 4096: ranges of 4096)
+    if tall and 16 < M <= K.TALL_MAX_ROWS and K_ % 8 == 0 and K._mid_fills_the_chip(N, K_, torch.device(DEV)):
+        assert parts.shape[0] == K._tall_plan(M, N, K_)[1] <= K.TALL_MAX_PARTS
+    elif 16 < M <= 64 and K_ % 8 == 0:   # K ranges of 1024 (up to 32 rows with K beyond 4096: ranges of 4096)
         assert parts.shape[0] == (-(-K_ // 4096) if M <= 32 and K_ > 4096 else -(-K_ // 1024))
         mid = K._gemm_mid(a.to(DEV), w.to(DEV), K_, False)   # not on this path, tested all the same
         _close(mid.sum(0), P.plain_linear(a.to(F64), w.to(F64)), 1e-5)
@@ -238,7 +244,7 @@ def test_gemm_split_over_k_and_its_consumer(K, monkeypatch, M, N, K_):
         assert K_ <= 4096 and M <= 16
         parts = parts[None]
     assert parts.dim() == 3 and parts.dtype == torch.float32
-    assert M > 16 or K_ <= 4096 or parts.shape[0] == -(-K_ // 4096)
+    assert M > 16 or K_ <= 4096 or parts.shape[0] == -(-K_ // 4096)   # up to 16 rows: K ranges of 4096
     want = P.plain_linear(a.to(F64), w.to(F64))
     _close(parts.sum(0), want, 1e-5)
     whole = K.gemm(a.to(DEV), w.to(DEV))
@@ -281,9 +287,13 @@ def test_swiglu_inside_the_down_projection(K, M, I, N):
                                          # 33 to 64 rows, and 17 to 32 with a long K: X through LDS
                                          (64, 16384, 4096, False), (33, 331, 1032, True), (48, 200, 96, False), (49, 4100, 520, True),
                                          (40, 5760, 2304, False), (64, 61, 8, True), (20, 96, 8200, False)])
-def test_gate_up_projection_with_the_activation_in_its_epilogue(K, monkeypatch, M, I, Kd, bias):
+@pytest.mark.parametrize("tall", [False, True])
+def test_gate_up_projection_with_the_activation_in_its_epilogue(K, monkeypatch, M, I, Kd, bias, tall):
     """One kernel for silu(x Wg^T) * (x Wu^T) against the plain formula and against the projection
-    followed by the activation kernel (gate and up rounded to bfloat16 at the same place)."""
+    followed by the activation kernel (gate and up rounded to bfloat16 at the same place).  `tall`: from 17 rows
+    the kernel with chunks of X in LDS where the outputs fill the chip; without it the kernels that keep X in
+    registers (up to 32 rows) or walk it through LDS in steps of 256 k (up to 64)."""
+    monkeypatch.setattr(K, "USE_TALL", tall)
     if I < 12288 and (M > 32 or (M > 16 and Kd > 4096)):
         # few outputs are left to the library on the engine's path (they do not fill the chip); the kernel is tested all the same
         assert K.gateup_swiglu_gemm(_rand((M, Kd), 31, torch.bfloat16).to(DEV), _rand((2 * I, Kd), 32, torch.bfloat16).to(DEV), None) is None
@@ -304,27 +314,25 @@ def test_gate_up_projection_with_the_activation_in_its_epilogue(K, monkeypatch, 
 
 
 @pytest.mark.parametrize("M,N,K_", [(17, 200, 264), (64, 128, 1024), (65, 334, 520), (100, 4096, 4096), (128, 130, 16384),
-                                    (129, 256, 640), (144, 4096, 16384), (208, 512, 2048), (97, 64, 72), (113, 1030, 4104)])
-def test_products_with_long_chunks_of_x_in_lds(K, monkeypatch, M, N, K_):
-    """`gemm_tall.hip`, both epilogues, weights in plain rows and in fragment order, against the plain formulas:
-    chunks of 512, 256 and 128 k (by the rows of X), K no multiple of a chunk, rows and outputs no multiple of a
-    tile, one part and many; and where the engine's path takes it."""
+                                    (129, 256, 640), (144, 4096, 16384), (208, 512, 2048), (97, 64, 72), (113, 1030, 4104),
+                                    (32, 4096, 16384), (48, 2304, 5760)])
+def test_products_with_chunks_of_x_in_lds(K, monkeypatch, M, N, K_):
+    """`gemm_tall.hip`, both epilogues, chunks of 64 and of 128 k, weights in plain rows and in fragment order, against
+    the plain formulas: K no multiple of a chunk, rows and outputs no multiple of a tile, one part and many."""
     from infinilm_amd.csrc import lib
     assert K.TALL_MAX_ROWS == lib.load().ilm_gemm_tall_max_rows()
-    assert all(K._tall_chunk(m) == lib.load().ilm_gemm_tall_chunk(m) for m in (17, 64, 65, 128, 129, 208))
     x, w = _rand((M, K_), 41, torch.bfloat16), _rand((N, K_), 42, torch.bfloat16, 0.05)
     want = P.plain_linear(x.to(F64), w.to(F64))
-    for fw in (None, K.pack_weight(w.to(DEV))):
-        parts = K._gemm_tall(x.to(DEV), w.to(DEV), K_, fw)
-        assert parts.dtype == torch.float32 and parts.shape == (K._tall_split(M, N, K_)[0], M, N)
-        _close(parts.sum(0), want, 1e-5)
-    if M > 64 and K._mid_fills_the_chip(N, K_, torch.device(DEV)):
-        took = []
-        monkeypatch.setattr(K, "_gemm_tall", lambda *a, **k: took.append("tall") or torch.zeros(1, M, N, device=DEV))
-        monkeypatch.setattr(K, "_gemm_mid", lambda *a, **k: took.append("mid") or torch.zeros(1, M, N, device=DEV))
-        K.gemm(x.to(DEV), w.to(DEV), allow_parts=True)
-        assert took == ["tall" if K._tall_chunks_per_part(M, N, K_) <= 4 or M >= K.TALL_LONG_K_MIN_ROWS else "mid"]
-        monkeypatch.undo()
+    kc, kb, cpp = K._tall_plan(M, N, K_)
+    assert kc in (64, 128) and kb <= K.TALL_MAX_PARTS and kb == -(-(-(-K_ // kc)) // cpp)
+    other = 192 - kc   # the other chunk length, split into three parts where there are that many chunks
+    chunks = -(-K_ // other)
+    cpp3 = -(-chunks // 3)
+    for plan in ((kc, kb, cpp), (other, -(-chunks // cpp3), cpp3)):
+        for fw in (None, K.pack_weight(w.to(DEV))):
+            parts = K._gemm_tall(x.to(DEV), w.to(DEV), K_, fw, plan)
+            assert parts.dtype == torch.float32 and parts.shape == (plan[1], M, N)
+            _close(parts.sum(0), want, 1e-5)
     inter = N // 2
     bias = _rand((2 * inter,), 43, torch.bfloat16, 0.1)
     wg = w[:2 * inter]
@@ -332,8 +340,8 @@ def test_products_with_long_chunks_of_x_in_lds(K, monkeypatch, M, N, K_):
     want_act = P.plain_swiglu(y[:, :inter], y[:, inter:])
     two = K.swiglu(K.gemm(x.to(DEV), wg.to(DEV), bias.to(DEV)))
     for fw in (None, K.pack_weight(wg.to(DEV), "gate_up8")):
-        for b in (bias.to(DEV), None):
-            act = K.gemm_tall_swiglu(x.to(DEV), wg.to(DEV), b, fw)
+        for b, kc_ in ((bias.to(DEV), 128), (bias.to(DEV), 64), (None, 128)):
+            act = K.gemm_tall_swiglu(x.to(DEV), wg.to(DEV), b, fw, kc_)
             assert act.shape == (M, inter) and act.dtype == torch.bfloat16
             if b is None:
                 y0 = P.plain_linear(x.to(F64), wg.to(F64))
@@ -344,12 +352,23 @@ def test_products_with_long_chunks_of_x_in_lds(K, monkeypatch, M, N, K_):
                 assert (act.float() - two.float()).abs().max() <= 2 ** -6 * max(float(two.float().abs().max()), 1e-6)
 
 
+def test_the_plan_of_a_product_with_parts():
+    """Chunks of 128 k and a workgroup a compute unit; chunks of 64 and two a unit where a part would be longer than
+    1024 k, up to 128 rows; never more than 16 parts."""
+    from infinilm_amd import kernels as K
+    assert K._tall_plan(64, 4096, 4096) == (128, 8, 4)       # o projection of the 8B shape: 32 tiles x 8 parts
+    assert K._tall_plan(64, 4096, 16384) == (64, 16, 16)     # down projection: 32 tiles x 16 parts of 1024 k
+    assert K._tall_plan(208, 4096, 16384) == (128, 8, 16)    # many rows: chunks of 128
+    assert K._tall_plan(64, 2304, 5760) == (128, 15, 3)
+    assert K._tall_plan(32, 128, 65536)[1] <= K.TALL_MAX_PARTS
+
+
 def test_where_the_gate_up_projection_keeps_x_in_lds(K, monkeypatch):
-    """65 to 112 rows, and up to 176 rows that are no multiple of 32, take the kernel with long chunks of X in LDS
+    """17 to 112 rows, and up to 176 rows that are no multiple of 32, take the kernel with chunks of X in LDS
     when the outputs fill the chip; other row counts are left to the library's product and the activation kernel."""
     monkeypatch.setattr(K, "GATEUP_WIDE_MIN_OUTPUTS", 0)
     w = _rand((2 * 96, 72), 44, torch.bfloat16, 0.1).to(DEV)
-    for M, taken in ((65, True), (96, True), (112, True), (113, True), (128, False), (144, True), (160, False), (176, True), (192, False),
+    for M, taken in ((17, True), (33, True), (65, True), (96, True), (112, True), (113, True), (128, False), (144, True), (160, False), (176, True), (192, False),
                      (175, True), (177, False), (208, False), (209, False)):
         x = _rand((M, 72), 45, torch.bfloat16).to(DEV)
         act = K.gateup_swiglu_gemm(x, w, None)
