@@ -190,6 +190,60 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __res
     }
 }
 
+// The same for few rows of bfloat16 activations whose branch comes in many float parts (the K-split products of a
+// decode step with 17 to 208 requests): a workgroup a row as above leaves most of the chip idle and walks the
+// parts in several rounds of loads; here 16 waves take a row, four columns a thread, and all parts' loads of a
+// thread (up to 16) are in flight at once.  The parts are summed in ascending order; the sum of squares is
+// reduced in an order that depends on H only (another one than the kernels above use: this one serves
+// bfloat16 activations only, where equal bits between the kernels are not promised).
+#define NORM_WIDE_THREADS 1024
+#define NORM_WIDE_PARTS 16
+template <typename WT>
+__global__ void __launch_bounds__(NORM_WIDE_THREADS)
+add_rmsnorm_wide_kernel(bf16* __restrict__ x, float* __restrict__ r, const float* __restrict__ h, const WT* __restrict__ w,
+                        int H, float alpha, float eps, int parts, size_t pstride, int frag_mg) {
+    __shared__ float red[NORM_WIDE_THREADS / 64];
+    const size_t base = (size_t)blockIdx.x * H;
+    const int j = threadIdx.x * 4;
+    const bool in = j < H;
+    const int jc = in ? j : 0;
+    float4 hv[NORM_WIDE_PARTS];
+#pragma unroll
+    for (int u = 0; u < NORM_WIDE_PARTS; ++u)
+        hv[u] = *reinterpret_cast<const float4*>(h + (size_t)(u < parts ? u : parts - 1) * pstride + base + jc);
+    float4 v = *reinterpret_cast<const float4*>(r + base + jc);
+    float wv[4];
+    if (sizeof(WT) == 2) {
+        const uint2 t = *reinterpret_cast<const uint2*>(w + jc);
+        wv[0] = __uint_as_float(t.x << 16); wv[1] = __uint_as_float(t.x & 0xffff0000u);
+        wv[2] = __uint_as_float(t.y << 16); wv[3] = __uint_as_float(t.y & 0xffff0000u);
+    } else {
+        const float4 t = *reinterpret_cast<const float4*>(w + jc);
+        wv[0] = t.x; wv[1] = t.y; wv[2] = t.z; wv[3] = t.w;
+    }
+    float4 hs = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int u = 0; u < NORM_WIDE_PARTS; ++u)
+        if (u < parts) { hs.x += hv[u].x; hs.y += hv[u].y; hs.z += hv[u].z; hs.w += hv[u].w; }
+    v.x += alpha * hs.x; v.y += alpha * hs.y; v.z += alpha * hs.z; v.w += alpha * hs.w;
+    if (in) *reinterpret_cast<float4*>(r + base + j) = v;
+    const float ss = in ? (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w) : 0.f;
+    const float tot = block_sum<NORM_WIDE_THREADS / 64>(ss, red);
+    const float rstd = 1.0f / sqrtf(tot / (float)H + eps);
+    bf16 o[4];
+    o[0] = from_f32<bf16>(v.x * rstd * wv[0]); o[1] = from_f32<bf16>(v.y * rstd * wv[1]);
+    o[2] = from_f32<bf16>(v.z * rstd * wv[2]); o[3] = from_f32<bf16>(v.w * rstd * wv[3]);
+    if (frag_mg > 0) {   // fragment order (frag.h): half of the 16-byte chunk of row blockIdx.x; zeros up to the next multiple of 32 k
+        const int kp = (H + 31) / 32 * 32;
+        if (j < kp) {
+            const uint2 val = in ? *reinterpret_cast<const uint2*>(o) : make_uint2(0u, 0u);
+            *reinterpret_cast<uint2*>(reinterpret_cast<bf16*>(x) + (size_t)frag_x_chunk(blockIdx.x, j >> 3, frag_mg) * 8 + (j & 7)) = val;
+        }
+    } else if (in) {
+        *reinterpret_cast<uint2*>(x + base + j) = *reinterpret_cast<const uint2*>(o);
+    }
+}
+
 // h: the pending branch [parts][rows][H] in the activations' dtype (h_dtype == dtype) or in float
 // (h_dtype == ILM_DTYPE_F32, e.g. the parts of a K-split product); null: nothing to add.
 extern "C" int ilm_add_rmsnorm(void* x, void* r, const void* h, const void* w, int rows, int H,
@@ -206,6 +260,18 @@ extern "C" int ilm_add_rmsnorm(void* x, void* r, const void* h, const void* w, i
                      ((uintptr_t)h & 15) == 0 && ((uintptr_t)w & 15) == 0 && pstride % 8 == 0;
     const int niter = (H + 2047) / 2048;
     const bool hf = h != nullptr && h_dtype == ILM_DTYPE_F32;
+    // few rows, many float parts, bfloat16 activations: the kernel with 16 waves a row
+    if (vec && hf && dtype == ILM_DTYPE_BF16 && parts >= 4 && parts <= NORM_WIDE_PARTS && rows <= 2 * ilm_num_cus() &&
+        H <= 4 * NORM_WIDE_THREADS && (H + 31) / 32 * 32 <= 4 * NORM_WIDE_THREADS) {
+        if (w_dtype == ILM_DTYPE_BF16)
+            add_rmsnorm_wide_kernel<bf16><<<rows, NORM_WIDE_THREADS, 0, stream>>>((bf16*)x, (float*)r, (const float*)h, (const bf16*)w, H, alpha, eps, parts, (size_t)pstride, frag_mg);
+        else if (w_dtype == ILM_DTYPE_F32)
+            add_rmsnorm_wide_kernel<float><<<rows, NORM_WIDE_THREADS, 0, stream>>>((bf16*)x, (float*)r, (const float*)h, (const float*)w, H, alpha, eps, parts, (size_t)pstride, frag_mg);
+        else
+            ILM_REQUIRE(false, "add_rmsnorm: unknown dtypes %d %d", dtype, w_dtype);
+        ILM_LAUNCH_CHECK("add_rmsnorm");
+        return 0;
+    }
 #define NORM_LAUNCH(T, WT, HT)                                                                                   \
     do {                                                                                                         \
         if (vec && niter <= 1)                                                                                   \

@@ -74,6 +74,32 @@ def test_add_rmsnorm(K, dtype, wdtype, H):
     assert torch.equal(x1.cpu(), x2[2:3].cpu())
 
 
+@pytest.mark.parametrize("rows,H,parts,wdtype", [(64, 4096, 16, torch.bfloat16), (33, 2304, 4, torch.float32), (5, 72, 7, torch.bfloat16),
+                                                 (208, 1032, 9, torch.bfloat16), (17, 4096, 3, torch.bfloat16), (40, 4104, 8, torch.bfloat16)])
+def test_add_rmsnorm_of_few_rows_with_many_float_parts(K, rows, H, parts, wdtype):
+    """The float32 parts of a K-split product into bfloat16 activations: 4 to 16 parts of rows up to 4096 wide take the
+    kernel with 16 waves a row (3 parts, or a wider row, the general one); plain rows and fragment order; the same
+    row gives the same bits whatever the rows around it."""
+    r = _rand((rows, H), 2, scale=3.0)
+    h = _rand((parts, rows, H), 3, scale=0.5)
+    w = _rand((H,), 4, wdtype) + 1
+    want_r = r.to(F64) + 0.37 * h.to(F64).sum(0)
+    want = P.plain_rmsnorm(want_r, w.to(F64), 1e-5)
+    rd = r.to(DEV).clone()
+    x = K.add_rmsnorm(rd, h.to(DEV), w.to(DEV), 0.37, 1e-5, torch.bfloat16)
+    _close(rd, want_r, 1e-6)
+    _close(x, want, 1e-2)
+    if rows <= K.FRAG_MAX_ROWS:
+        rd2 = r.to(DEV).clone()
+        xf = K.add_rmsnorm(rd2, h.to(DEV), w.to(DEV), 0.37, 1e-5, torch.bfloat16, frag=True)
+        assert torch.equal(rd2, rd) and torch.equal(K.from_frag(xf), x)
+        if H % 32:   # the k up to the next multiple of 32 are zeros in fragment order
+            raw = xf.data.view(torch.bfloat16).view(-(-H // 32), -(-rows // 16), 4, 16, 8).cpu()
+            assert not raw[-1, :, (H % 32) // 8:].any()
+    one = K.add_rmsnorm(r[3:4].to(DEV).clone(), h[:, 3:4].contiguous().to(DEV), w.to(DEV), 0.37, 1e-5, torch.bfloat16)
+    assert torch.equal(one, x[3:4])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nh,nkv,d,rd,page", [(4, 2, 16, 16, 4), (3, 1, 48, 48, 16), (5, 5, 32, 16, 8), (2, 1, 80, 0, 16)])
 def test_rope_and_cache_write(K, dtype, nh, nkv, d, rd, page):
