@@ -28,9 +28,7 @@ _SIGNATURES = {
     "ilm_scale_rows": [_P, _I, _I, _I, _F, _P],
     "ilm_gemm_gateup_swiglu": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _I, _P, _I, _F, _P],
     "ilm_gemm_tail": [_P, _I, _P, _I, _P, _P, _I, _P, _I, _P, _P, _I, _F, _I, _I, _I, _P],
-    "ilm_gemm_gateup_wide": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _P],
     "ilm_gemm_rows64": [_P, _I, _L, _I, _P, _I, _I, _I, _I, _P, _I, _I, _P],
-    "ilm_gemm_mid": [_P, _I, _L, _I, _I, _P, _I, _I, _I, _I, _P, _I, _I, _P],
     "ilm_gemm_tall": [_P, _I, _L, _I, _I, _I, _P, _I, _I, _I, _I, _P, _I, _I, _P],
     "ilm_gemm_tall_swiglu": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "ilm_gemm_qkv_rope": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],

@@ -313,21 +313,18 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
     aligned = K % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 \
         and w.data_ptr() % 16 == 0
     plain = bias is None and alpha == 1.0
-    # 65 to 208 rows on their way into the residual sum: split over K, where the vendor library leaves the
-    # chip idle (measured at the 8B shapes: down projection 68 -> 36 us at 96 rows, 81 -> 39 at 128, 92 -> 44
-    # at 160, 114 -> 48 at 192, 63 -> 51 at 208; o projection 22 -> 17, 25 -> 19, 32 -> 23 at 192)
-    # (not for small matrices, whose few tiles leave most of the chip idle whatever the split: 0.5B shape at 128
-    # rows 2.22 against 1.96 ms a step with the library)
+    # (From 65 rows on the vendor library leaves the chip idle on such products: down projection 68 us at 96 rows, 81
+    # at 128, 92 at 160, 114 at 192, 63 at 208; o projection 22, 25, 32 at 192.  Not for small matrices, whose few
+    # tiles leave most of the chip idle whatever the split: 0.5B shape at 128 rows 2.22 against 1.96 ms a step with
+    # the library.)
     # 17 to 208 rows on their way into the residual sum: chunks of X resident in LDS, two workgroups a compute unit
     # (gemm_tall.hip).  Measured at the 8B shapes against the kernels it took over from: o projection 9.8 us against
-    # 10.6 (K ranges of 1024, X in registers) at 32 rows, 11.0 / 12.4 at 64, 12.8 / 17.1 (steps of 64 k, X through LDS)
-    # at 96, 15.8 / 19.4 at 128, 16.9 / 22.2 at 160; down projection 27.7 / 33.1 (four parts of 4096, X in registers) at
+    # 10.6 (K ranges of 1024, X in registers) at 32 rows, 11.0 / 12.4 at 64, 12.8 / 17.1 (steps of 64 k, X through LDS, a
+    # step's loads waited for before the next step's were issued) at 96, 15.8 / 19.4 at 128, 16.9 / 22.2 at 160; down projection 27.7 / 33.1 (four parts of 4096, X in registers) at
     # 32 rows, 30.3 / 33.3 at 64, 33.7 / 38.1 at 96, 37.1 / 42.0 at 128, 46.2 / 47.1 at 160, 52.0 / 56.7 at 208
     if (fast and aligned and plain and allow_parts and out is None and USE_TALL and TALL_MIN_ROWS <= M <= TALL_MAX_ROWS
-            and M > 16 and _mid_fills_the_chip(N, K, a.device)):
+            and M > 16 and _tall_fills_the_chip(N, K, a.device)):
         return _gemm_tall(a, w, K, frag_w)
-    if fast and aligned and plain and allow_parts and out is None and 64 < M <= MID_MAX_ROWS and _mid_fills_the_chip(N, K, a.device):
-        return _gemm_mid(a, w, K, False)
     # 17 to 64 rows on their way into the residual sum: K in ranges of 1024 with the X fragments of all rows
     # in registers (o projection at 64 rows 13.1 against the library's 18.9 us, down projection 33.9
     # against 41.3, of which the sum of its 16 parts takes 5 back; up to 32 rows the down projection
@@ -408,31 +405,15 @@ F32_FEW_ROWS = int(os.environ.get("INFINILM_AMD_F32_FEW_ROWS", "64"))
 
 ROWS64_SPAN = 1024   # K range of one part of the 17-to-64-rows product (ilm_gemm_rows64_span())
 ROWS64_MAX_PARTS = int(os.environ.get("INFINILM_AMD_ROWS64_PARTS", "16"))   # 0: never this kernel
-MID_MAX_ROWS = int(os.environ.get("INFINILM_AMD_MID_ROWS", "208"))  # 16: above 16 rows always the library
-MID_MIN_WGS_PER_CU = 0.25   # the medium-rows product is used where its grid can give more than a quarter of the units a workgroup
+TALL_MIN_WGS_PER_CU = 0.25   # the tall product is used where its grid can give more than a quarter of the units a workgroup
 
 
-def _mid_fills_the_chip(N: int, K: int, device) -> bool:
-    """The medium-rows product cuts W into tiles of 128 rows and K into ranges of at least 512: with fewer
-    workgroups than a quarter of the compute units whatever the split, the vendor library's product is faster
-    (measured: the 0.5B shape's 1024 x 4096 gives 64 workgroups on 256 units and loses, 2.22 against 1.96 ms a step
-    at 128 rows; the 2B-family's 2304 x 2304 gives 72 and wins)."""
-    return -(-N // 128) * max(K // 512, 1) > MID_MIN_WGS_PER_CU * _num_cus(device)
-MID_TARGET_WGS = int(os.environ.get("INFINILM_AMD_MID_WGS", "512"))
-
-
-def _gemm_mid(x: torch.Tensor, w: torch.Tensor, K: int, act: bool) -> torch.Tensor:
-    """17 to 128 rows, result in float32 parts [P, M, N] split over K (see gemm_mid.hip); `act`: x holds
-    rows [gate | up] and the product takes silu(gate) * up."""
-    M, N = x.shape[0], w.shape[0]
-    n_tiles = -(-N // 128)
-    kb = max(1, min(-(-MID_TARGET_WGS // n_tiles), K // 512 or 1))
-    kspan = -(-K // (kb * 128)) * 128
-    kb = -(-K // kspan)
-    parts = torch.empty((kb, M, N), dtype=F32, device=x.device)
-    _run("ilm_gemm_mid", parts.data_ptr(), N, M * N, kb, kspan, w.data_ptr(), w.stride(0), M, N, K, x.data_ptr(),
-         x.stride(0), 1 if act else 0, _stream())
-    return parts
+def _tall_fills_the_chip(N: int, K: int, device) -> bool:
+    """The tall product cuts W into tiles of 128 rows and K into ranges of at least 512: with fewer workgroups
+    than a quarter of the compute units whatever the split, the vendor library's product is faster (measured with
+    the kernel this one replaced, which cut alike: the 0.5B shape's 1024 x 4096 gives 64 workgroups on 256 units and
+    loses, 2.22 against 1.96 ms a step at 128 rows; the 2B-family's 2304 x 2304 gives 72 and wins)."""
+    return -(-N // 128) * max(K // 512, 1) > TALL_MIN_WGS_PER_CU * _num_cus(device)
 
 
 USE_TALL = os.environ.get("INFINILM_AMD_TALL", "1") == "1"
@@ -493,9 +474,8 @@ def gemm_tall_swiglu(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
 
 
 USE_GATEUP_SWIGLU = os.environ.get("INFINILM_AMD_GATEUP_SWIGLU", "1") == "1"
-USE_GATEUP_WIDE = os.environ.get("INFINILM_AMD_GATEUP_WIDE", "1") == "1"
-# outputs from which the kernel with X through LDS is used (-1: 48 a compute unit; 0: always, as its tests do)
-GATEUP_WIDE_MIN_OUTPUTS = int(os.environ.get("INFINILM_AMD_GATEUP_WIDE_MIN", "-1"))
+# outputs from which the gate/up kernel with X in LDS is used (-1: 48 a compute unit; 0: always, as its tests do)
+GATEUP_TALL_MIN_OUTPUTS = int(os.environ.get("INFINILM_AMD_GATEUP_TALL_MIN", "-1"))
 
 
 # Rows up to which the projection that ends a branch takes the residual sum and the first half of the next
@@ -550,9 +530,9 @@ def gateup_resident_ok(rows: int, w: torch.Tensor) -> bool:
 def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
                        row_ss: Optional[torch.Tensor] = None, eps: float = 0.0, frag_w=None) -> Optional[torch.Tensor]:
     """silu(x Wg^T + bg) * (x Wu^T + bu) for few rows in bfloat16, W = [Wg; Wu]: the fused gate/up
-    projection with the SwiGLU in its epilogue, [M, I] (up to 32 rows with X in registers, up to 64 with X
-    through LDS).  None where no kernel applies (more rows, float32): the caller then runs the projection
-    and the activation.  `row_ss`: x is what `gemm_tail` left (residual * norm weight) and row_ss its
+    projection with the SwiGLU in its epilogue, [M, I] (up to 32 rows with X in registers; 17 to 208 with chunks
+    of X in LDS where the outputs fill the chip).  None where no kernel applies (more rows, few outputs,
+    float32): the caller then runs the projection and the activation.  `row_ss`: x is what `gemm_tail` left (residual * norm weight) and row_ss its
     partial sums of squares: the rows' division by sqrt(mean square + eps) happens in this kernel's
     epilogue (only the kernel with X in registers does that: `gateup_resident_ok`)."""
     M, K = x.shape
@@ -561,21 +541,19 @@ def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
         if not (resident and gateup_resident_ok(M, w) and _mfma_operands_ok(x, w, K) and row_ss.dtype == F32
                 and row_ss.dim() == 2 and row_ss.shape[1] == TAIL_SS_ROWS and row_ss.is_contiguous() and row_ss.is_cuda):
             raise KernelError("a product with the norm's division in its epilogue needs the few-rows gate/up kernel")
-    # 17 to 64 rows that do not fit the registers: X through LDS, W streamed over the whole K by every wave
-    # (64 rows at the 8B shape: 52 us against 62 + 5 for the vendor library's product and the activation kernel)
     # (a workgroup takes 64 outputs: with fewer outputs than three quarters of the compute units have workgroups
-    # the library is faster - 2B-family shape, 5,760 outputs, 64 rows: 6.40 against 6.07 ms a step)
-    wide_min = GATEUP_WIDE_MIN_OUTPUTS if GATEUP_WIDE_MIN_OUTPUTS >= 0 else 48 * _num_cus(x.device)
-    wide = USE_GATEUP_WIDE and not resident and 16 < M <= 64 and w.shape[0] // 2 >= wide_min
+    # the library is faster - measured with the kernel this one replaced, which cut alike: 2B-family shape, 5,760
+    # outputs, 64 rows: 6.40 against 6.07 ms a step)
+    tall_min = GATEUP_TALL_MIN_OUTPUTS if GATEUP_TALL_MIN_OUTPUTS >= 0 else 48 * _num_cus(x.device)
     # 17 to 112 rows, and up to 176 where the rows are no multiple of 32 (the vendor library's product is then slow):
     # chunks of X resident in LDS, two workgroups a compute unit (gemm_tall.hip).  Measured at the 8B shape: 48.1 us
     # against 52.9 (X in registers, two row groups) at 32 rows, 53.2 against 57.4 (X through LDS in steps of 256 k, one
-    # workgroup a unit) at 64; against the library's product and the activation kernel 57.7 / 66.2 at 96, 66.5 / 81.4 at
+    # workgroup a unit: the kernel it replaced) at 64; against the library's product and the activation kernel 57.7 / 66.2 at 96, 66.5 / 81.4 at
     # 112, 71.2 / 69.0 at 128, 76.1 / 85.2 at 144, 75.3 / 72.7 at 160, 82.8 / 90.1 at 176, 86.6 / 75.6 at 192, 90.4 / 83.0 at 208
-    tall = (USE_TALL and USE_GATEUP_WIDE and row_ss is None and max(TALL_MIN_ROWS, 17) <= M <= TALL_MAX_ROWS
-            and w.shape[0] // 2 >= wide_min and (M <= TALL_GATEUP_MAX_ROWS or (M % 32 != 0 and M <= 176)))
+    tall = (USE_TALL and row_ss is None and max(TALL_MIN_ROWS, 17) <= M <= TALL_MAX_ROWS
+            and w.shape[0] // 2 >= tall_min and (M <= TALL_GATEUP_MAX_ROWS or (M % 32 != 0 and M <= 176)))
     if not (USE_GATEUP_SWIGLU and not FORCE_BASIC and x.dtype == BF16 and w.dtype == BF16 and x.is_cuda
-            and (resident or wide or tall) and K % 8 == 0 and w.shape[0] % 2 == 0 and w.shape[1] == K
+            and (resident or tall) and K % 8 == 0 and w.shape[0] % 2 == 0 and w.shape[1] == K
             and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         return None
@@ -586,17 +564,8 @@ def gateup_swiglu_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Te
     if tall:
         return gemm_tall_swiglu(x, w, bias, frag_w)
     out = torch.empty((M, I), dtype=BF16, device=x.device)
-    if resident:
-        _run("ilm_gemm_gateup_swiglu", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
-             _ptr(bias), M, I, K, _ptr(row_ss), 0 if row_ss is None else row_ss.shape[0], float(eps), _stream())
-    else:
-        fw = _frag_of(frag_w) if USE_FRAG else None
-        if fw is not None:   # W in fragment order (tiles of 8 gate + 8 up rows): 64.1 -> 56.8 us at 64 rows of the 8B shape
-            _run("ilm_gemm_gateup_wide", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), fw.data.data_ptr(), 0,
-                 _ptr(bias), M, I, K, 1, _stream())
-        else:
-            _run("ilm_gemm_gateup_wide", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
-                 _ptr(bias), M, I, K, 0, _stream())
+    _run("ilm_gemm_gateup_swiglu", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0),
+         _ptr(bias), M, I, K, _ptr(row_ss), 0 if row_ss is None else row_ss.shape[0], float(eps), _stream())
     return out
 
 
@@ -607,7 +576,7 @@ def swiglu_gemm(gate_up: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor
     K = two_k // 2
     N = w.shape[0]
     # (above 32 rows the activation would be recomputed by every workgroup along N: the separate kernel
-    # and the medium-rows product are faster, 38 against 42 us at 64 rows)
+    # and the product with parts are faster, 38 against 42 us at 64 rows)
     ok = (gate_up.dtype == BF16 and w.dtype == BF16 and not FORCE_BASIC and USE_KSPLIT and M <= max(16, FEW_ROWS)
           and two_k % 2 == 0
           and w.shape[1] == K and K % 8 == 0 and gate_up.stride(1) == 1 and w.stride(1) == 1 and gate_up.stride(0) % 8 == 0
@@ -645,7 +614,7 @@ def bound_pages(need: int) -> int:
 def bound_rows(rows: int) -> int:
     """The number of rows a decode step of `rows` requests is served with when it is recorded: 1, 2, 4, 8,
     16, 24, 32, 48, 64, 96, 128, 160, 208, 256, 384, 512, ... (the rest are rows of no request).  The sizes end
-    where the products change kernels (16, 32, 64 rows; 208, the last size of the medium-rows product), so a
+    where the products change kernels (16, 32, 64 rows; 208, the last size of the product with chunks of X in LDS), so a
     filled-up step runs the kernels the step itself would run and its recording equals the eager step."""
     for b in (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 160, 208, 256):
         if rows <= b:

@@ -254,18 +254,17 @@ def test_gemm_split_over_k_and_its_consumer(K, monkeypatch, M, N, K_, tall):
     that serve when it is switched off."""
     monkeypatch.setattr(K, "USE_TALL", tall)
     a, w = _rand((M, K_), 14, torch.bfloat16), _rand((N, K_), 15, torch.bfloat16, 0.05)
-    small = M > 64 and not K._mid_fills_the_chip(N, K_, torch.device(DEV))
-    if small:
-        # a small matrix is left to the library on the engine's path; the medium-rows kernel is tested all the same
+    if M > 64 and not (tall and K._tall_fills_the_chip(N, K_, torch.device(DEV))):
+        # many rows of a small matrix (or without that product) are left to the library on the engine's path
         assert K.gemm(a.to(DEV), w.to(DEV), allow_parts=True).dtype == torch.bfloat16
-        monkeypatch.setattr(K, "MID_MIN_WGS_PER_CU", -1.0)
+        if not tall:
+            return
+        monkeypatch.setattr(K, "TALL_MIN_WGS_PER_CU", -1.0)   # the kernel is tested all the same
     parts = K.gemm(a.to(DEV), w.to(DEV), allow_parts=True)
-    if tall and 16 < M <= K.TALL_MAX_ROWS and K_ % 8 == 0 and K._mid_fills_the_chip(N, K_, torch.device(DEV)):
+    if tall and 16 < M <= K.TALL_MAX_ROWS and K_ % 8 == 0 and K._tall_fills_the_chip(N, K_, torch.device(DEV)):
         assert parts.shape[0] == K._tall_plan(M, N, K_)[1] <= K.TALL_MAX_PARTS
     elif 16 < M <= 64 and K_ % 8 == 0:   # K ranges of 1024 (up to 32 rows with K beyond 4096: ranges of 4096)
         assert parts.shape[0] == (-(-K_ // 4096) if M <= 32 and K_ > 4096 else -(-K_ // 1024))
-        mid = K._gemm_mid(a.to(DEV), w.to(DEV), K_, False)   # not on this path, tested all the same
-        _close(mid.sum(0), P.plain_linear(a.to(F64), w.to(F64)), 1e-5)
     if parts.dim() == 2:   # short K and few rows: one float32 result
         assert K_ <= 4096 and M <= 16
         parts = parts[None]
@@ -289,20 +288,17 @@ def test_gemm_split_over_k_and_its_consumer(K, monkeypatch, M, N, K_, tall):
     _close(x, P.plain_rmsnorm(want_r, nw.to(F64), 1e-6), 1e-2)
 
 
-@pytest.mark.parametrize("M,I,N", [(8, 16384, 4096), (3, 200, 96), (16, 4104, 50), (17, 4104, 50), (40, 8192, 1024),
-                                   (64, 16384, 4096), (33, 96, 331), (128, 1000, 70), (100, 16384, 4096), (32, 16384, 4096),
-                                   (24, 200, 96)])
+@pytest.mark.parametrize("M,I,N", [(8, 16384, 4096), (3, 200, 96), (16, 4104, 50), (17, 4104, 50), (32, 16384, 4096),
+                                   (24, 200, 96), (33, 96, 331)])
 def test_swiglu_inside_the_down_projection(K, M, I, N):
     gu = _rand((M, 2 * I), 18, torch.bfloat16, 1.5)
     w = _rand((N, I), 19, torch.bfloat16, 0.05)
-    if M <= 32:
-        parts = K.swiglu_gemm(gu.to(DEV), w.to(DEV))
-    else:   # the medium-rows kernel's variant with the activation on the way into LDS (not on the engine's path)
+    if M > 32:   # more rows: the activation kernel and a product of its own
         assert K.swiglu_gemm(gu.to(DEV), w.to(DEV)) is None
-        parts = K._gemm_mid(gu.to(DEV), w.to(DEV), I, True)
+        return
+    parts = K.swiglu_gemm(gu.to(DEV), w.to(DEV))
     assert parts is not None and parts.dtype == torch.float32 and parts.shape[1:] == (M, N)
-    if M <= 32:
-        assert parts.shape[0] == -(-I // 4096)
+    assert parts.shape[0] == -(-I // 4096)
     act = P.plain_swiglu(gu.to(F64)[:, :I], gu.to(F64)[:, I:])
     _close(parts.sum(0), P.plain_linear(act, w.to(F64)), 6e-3)   # the activation is rounded to bfloat16 once
 
@@ -310,20 +306,23 @@ def test_swiglu_inside_the_down_projection(K, M, I, N):
 @pytest.mark.parametrize("M,I,Kd,bias", [(8, 16384, 4096, False), (3, 200, 96, True), (16, 331, 1032, False), (17, 331, 1032, True),
                                          (32, 4096, 4096, False), (5, 50, 8192, True), (24, 96, 200, False),
                                          (20, 8200, 1032, True), (2, 5760, 2304, False),
-                                         # 33 to 64 rows, and 17 to 32 with a long K: X through LDS
+                                         # 33 to 64 rows, and 17 to 32 with a long K: chunks of X in LDS
                                          (64, 16384, 4096, False), (33, 331, 1032, True), (48, 200, 96, False), (49, 4100, 520, True),
                                          (40, 5760, 2304, False), (64, 61, 8, True), (20, 96, 8200, False)])
 @pytest.mark.parametrize("tall", [False, True])
 def test_gate_up_projection_with_the_activation_in_its_epilogue(K, monkeypatch, M, I, Kd, bias, tall):
     """One kernel for silu(x Wg^T) * (x Wu^T) against the plain formula and against the projection
     followed by the activation kernel (gate and up rounded to bfloat16 at the same place).  `tall`: from 17 rows
-    the kernel with chunks of X in LDS where the outputs fill the chip; without it the kernels that keep X in
-    registers (up to 32 rows) or walk it through LDS in steps of 256 k (up to 64)."""
+    the kernel with chunks of X in LDS where the outputs fill the chip; without it the kernel that keeps X in
+    registers (up to 32 rows of a K up to 4096)."""
     monkeypatch.setattr(K, "USE_TALL", tall)
-    if I < 12288 and (M > 32 or (M > 16 and Kd > 4096)):
-        # few outputs are left to the library on the engine's path (they do not fill the chip); the kernel is tested all the same
-        assert K.gateup_swiglu_gemm(_rand((M, Kd), 31, torch.bfloat16).to(DEV), _rand((2 * I, Kd), 32, torch.bfloat16).to(DEV), None) is None
-        monkeypatch.setattr(K, "GATEUP_WIDE_MIN_OUTPUTS", 0)
+    if M > 32 or (M > 16 and Kd > 4096):   # rows that do not fit the registers
+        if I < 12288 or not tall:
+            # few outputs are left to the library on the engine's path (they do not fill the chip)
+            assert K.gateup_swiglu_gemm(_rand((M, Kd), 31, torch.bfloat16).to(DEV), _rand((2 * I, Kd), 32, torch.bfloat16).to(DEV), None) is None
+        if not tall:
+            return
+        monkeypatch.setattr(K, "GATEUP_TALL_MIN_OUTPUTS", 0)   # the kernel is tested all the same
     x, w = _rand((M, Kd), 31, torch.bfloat16), _rand((2 * I, Kd), 32, torch.bfloat16, scale=2.0 * Kd ** -0.5)
     b = _rand((2 * I,), 33, torch.bfloat16) if bias else None
     dev = lambda t: None if t is None else t.to(DEV)
@@ -392,7 +391,7 @@ def test_the_plan_of_a_product_with_parts():
 def test_where_the_gate_up_projection_keeps_x_in_lds(K, monkeypatch):
     """17 to 112 rows, and up to 176 rows that are no multiple of 32, take the kernel with chunks of X in LDS
     when the outputs fill the chip; other row counts are left to the library's product and the activation kernel."""
-    monkeypatch.setattr(K, "GATEUP_WIDE_MIN_OUTPUTS", 0)
+    monkeypatch.setattr(K, "GATEUP_TALL_MIN_OUTPUTS", 0)
     w = _rand((2 * 96, 72), 44, torch.bfloat16, 0.1).to(DEV)
     for M, taken in ((17, True), (33, True), (65, True), (96, True), (112, True), (113, True), (128, False), (144, True), (160, False), (176, True), (192, False),
                      (175, True), (177, False), (208, False), (209, False)):
