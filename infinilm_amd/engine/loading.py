@@ -63,11 +63,37 @@ def load_model(model_dir: str, dtype=None, device="cuda:0") -> CausalLM:
     return model
 
 
+def fragment_copy_bytes(model: CausalLM) -> int:
+    """Bytes the projections' second copies in fragment order take once every product has packed its own: they are
+    made at a product's first use with 17 or more rows (`FusedLinear.frag_weight`), long after the cache pool has
+    been sized, so the pool leaves room for them."""
+    from .. import kernels
+    from ..parts.linear import FusedLinear
+    total, seen, stack = 0, set(), [model]
+    while stack:
+        o = stack.pop()
+        if id(o) in seen:
+            continue
+        seen.add(id(o))
+        if isinstance(o, FusedLinear):
+            if kernels.frag_weight_ok(o.weight):
+                total += o.weight.numel() * o.weight.element_size()
+        elif isinstance(o, (list, tuple)):
+            stack.extend(o)
+        elif isinstance(o, dict):
+            stack.extend(o.values())
+        elif type(o).__module__.startswith("infinilm_amd") and hasattr(o, "__dict__"):
+            stack.extend(vars(o).values())
+    return total
+
+
 def pages_that_fit(model: CausalLM, page_size: int, memory_fraction: float = 0.9, reserve_bytes: int = 4 << 30) -> int:
     """Pages per group that `memory_fraction` of the device's free memory holds (after `reserve_bytes`
-    for activations, graphs and workspaces), for `num_pages=None`: the cache takes what the weights
-    leave, on a 288 GB part some hundred thousand tokens for a model of this size."""
+    for activations, graphs and workspaces, and after the weights' copies in fragment order that are still to
+    be made), for `num_pages=None`: the cache takes what the weights leave, on a 288 GB part some hundred
+    thousand tokens for a model of this size."""
     from ..cache.needs import PagedKV
+    reserve_bytes += fragment_copy_bytes(model)
     elem = torch.empty((), dtype=model.dtype).element_size()
     per_page = sum(2 * n.num_kv_heads * n.head_dim * page_size * elem for n in model.cache_needs if isinstance(n, PagedKV))
     if per_page == 0:
