@@ -192,13 +192,13 @@ add_rmsnorm_vec_kernel(T* __restrict__ x, float* __restrict__ r, const HT* __res
 
 // The same for few rows of bfloat16 activations whose branch comes in many float parts (the K-split products of a
 // decode step with 17 to 208 requests): a workgroup a row as above leaves most of the chip idle and walks the
-// parts in several rounds of loads; here 16 waves take a row, four columns a thread, and all parts' loads of a
-// thread (up to 16) are in flight at once.  The parts are summed in ascending order; the sum of squares is
+// parts in several rounds of loads; here up to 16 waves take a row (as many as its width gives four columns a
+// thread), and all parts' loads of a thread (up to 16) are in flight at once.  The parts are summed in ascending order; the sum of squares is
 // reduced in an order that depends on H only (another one than the kernels above use: this one serves
 // bfloat16 activations only, where equal bits between the kernels are not promised).
 #define NORM_WIDE_THREADS 1024
 #define NORM_WIDE_PARTS 16
-template <typename WT>
+template <typename WT, int PB>   // PB: slots for parts (8 or 16; slots beyond the parts load the last part again)
 __global__ void __launch_bounds__(NORM_WIDE_THREADS)
 add_rmsnorm_wide_kernel(bf16* __restrict__ x, float* __restrict__ r, const float* __restrict__ h, const WT* __restrict__ w,
                         int H, float alpha, float eps, int parts, size_t pstride, int frag_mg) {
@@ -207,9 +207,9 @@ add_rmsnorm_wide_kernel(bf16* __restrict__ x, float* __restrict__ r, const float
     const int j = threadIdx.x * 4;
     const bool in = j < H;
     const int jc = in ? j : 0;
-    float4 hv[NORM_WIDE_PARTS];
+    float4 hv[PB];
 #pragma unroll
-    for (int u = 0; u < NORM_WIDE_PARTS; ++u)
+    for (int u = 0; u < PB; ++u)
         hv[u] = *reinterpret_cast<const float4*>(h + (size_t)(u < parts ? u : parts - 1) * pstride + base + jc);
     float4 v = *reinterpret_cast<const float4*>(r + base + jc);
     float wv[4];
@@ -223,12 +223,17 @@ add_rmsnorm_wide_kernel(bf16* __restrict__ x, float* __restrict__ r, const float
     }
     float4 hs = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-    for (int u = 0; u < NORM_WIDE_PARTS; ++u)
+    for (int u = 0; u < PB; ++u)
         if (u < parts) { hs.x += hv[u].x; hs.y += hv[u].y; hs.z += hv[u].z; hs.w += hv[u].w; }
     v.x += alpha * hs.x; v.y += alpha * hs.y; v.z += alpha * hs.z; v.w += alpha * hs.w;
     if (in) *reinterpret_cast<float4*>(r + base + j) = v;
     const float ss = in ? (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w) : 0.f;
-    const float tot = block_sum<NORM_WIDE_THREADS / 64>(ss, red);
+    // over the block's waves, in wave order (their number follows from H alone)
+    float tot = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = tot;
+    __syncthreads();
+    tot = 0.f;
+    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) tot += red[i];
     const float rstd = 1.0f / sqrtf(tot / (float)H + eps);
     bf16 o[4];
     o[0] = from_f32<bf16>(v.x * rstd * wv[0]); o[1] = from_f32<bf16>(v.y * rstd * wv[1]);
@@ -263,11 +268,14 @@ extern "C" int ilm_add_rmsnorm(void* x, void* r, const void* h, const void* w, i
     // few rows, many float parts, bfloat16 activations: the kernel with 16 waves a row
     if (vec && hf && dtype == ILM_DTYPE_BF16 && parts >= 4 && parts <= NORM_WIDE_PARTS && rows <= 2 * ilm_num_cus() &&
         H <= 4 * NORM_WIDE_THREADS && (H + 31) / 32 * 32 <= 4 * NORM_WIDE_THREADS) {
-        if (w_dtype == ILM_DTYPE_BF16)
-            add_rmsnorm_wide_kernel<bf16><<<rows, NORM_WIDE_THREADS, 0, stream>>>((bf16*)x, (float*)r, (const float*)h, (const bf16*)w, H, alpha, eps, parts, (size_t)pstride, frag_mg);
-        else if (w_dtype == ILM_DTYPE_F32)
-            add_rmsnorm_wide_kernel<float><<<rows, NORM_WIDE_THREADS, 0, stream>>>((bf16*)x, (float*)r, (const float*)h, (const float*)w, H, alpha, eps, parts, (size_t)pstride, frag_mg);
-        else
+        const int threads = (((H + 31) / 32 * 32 / 4) + 63) / 64 * 64;   // four columns a thread, whole waves
+#define NORM_WIDE(WT, PB) add_rmsnorm_wide_kernel<WT, PB><<<rows, threads, 0, stream>>>((bf16*)x, (float*)r, (const float*)h, (const WT*)w, H, alpha, eps, parts, (size_t)pstride, frag_mg)
+        if (w_dtype == ILM_DTYPE_BF16) {
+            if (parts <= 8) NORM_WIDE(bf16, 8); else NORM_WIDE(bf16, 16);
+        } else if (w_dtype == ILM_DTYPE_F32) {
+            if (parts <= 8) NORM_WIDE(float, 8); else NORM_WIDE(float, 16);
+        } else
+#undef NORM_WIDE
             ILM_REQUIRE(false, "add_rmsnorm: unknown dtypes %d %d", dtype, w_dtype);
         ILM_LAUNCH_CHECK("add_rmsnorm");
         return 0;
