@@ -154,8 +154,12 @@ def main(argv=None) -> int:
     try:
         if cfg.warmup:
             print("=================== warmup start ===================", flush=True)
-            for c in cases:   # also records the HIP graphs of each batch size
-                run_case(llm, dict(c, output_len=min(c["output_len"], 4)), cfg.seed, sp_kwargs)
+            # with graphs a step's shape is recorded the second time it comes: the warm-up runs each case twice, so that
+            # the prompts' steps of the measured run are replays and not recordings
+            # (prompts of its own for each pass: with prefix caching a prompt that comes again is not computed again)
+            for rep in range(2 if cfg.enable_graph else 1):
+                for c in cases:
+                    run_case(llm, dict(c, output_len=min(c["output_len"], 4)), cfg.seed + 500 * rep, sp_kwargs)
             print("=================== warmup done ====================", flush=True)
         for i, c in enumerate(cases):   # prompts of their own for every case: no case finds another's pages
             print(json.dumps(run_case(llm, c, cfg.seed + 1 + 1000 * (i + 1), sp_kwargs)), flush=True)

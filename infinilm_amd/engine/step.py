@@ -82,6 +82,7 @@ class StepRunner:
         # take their indices from the device's tensors in such steps
         self.graph_mixed = all(getattr(b, "records_mixed_steps", False) for b in getattr(model, "blocks", []))
         self.graph_mixed_max_tokens = 8192   # ... up to this many tokens a step (a recording keeps the step's activations)
+        self.graph_mixed_pad_share = 8       # ... whose bounded shape adds at most 1/8 of rows of no request (0: any)
         self._pinned: List[Optional[torch.Tensor]] = [None, None]   # two staging buffers in turn
         self._copy_done: List[Optional[torch.cuda.Event]] = [None, None]
         self._stage_turn = 0
@@ -430,11 +431,14 @@ class StepRunner:
         """The bounded shape of a step that holds portions of prompts (and decoded tokens beside them): tokens, requests,
         wanted rows and block-table width, each rounded up (`kernels.bound_rows`, `kernels.bound_pages`); the lists of
         attention tiles and of single rows are as long as those allow.  Under a token budget the steps of a busy engine have the budget's tokens and differ in
-        the rest by little, so few shapes serve them.  None: not recorded (too many tokens)."""
+        the rest by little, so few shapes serve them.  None: not recorded (too many tokens, or a token count that its
+        bound would fill up by more than an eighth: a prompt of 1,100 tokens alone would run as 1,536 rows)."""
         cache = self.cache
         T = sum(len(e.tokens) for e in entries)
         if T > self.graph_mixed_max_tokens:
             return None
+        if self.graph_mixed_pad_share and kernels.bound_rows(T) - T > T // self.graph_mixed_pad_share:
+            return None   # the rows that fill the shape up are computed too: more than an eighth of them is not worth a replay
         n_want = sum(len(e.want) for e in entries)
         need = max(-(-(cache.length(e.req_id) + len(e.tokens)) // cache.page_size) for e in entries)
         return self._mixed_shape(kernels.bound_rows(T), n_want, any(len(e.tokens) == 1 for e in entries), need)

@@ -866,6 +866,7 @@ def test_recorded_steps_with_portions_of_prompts(models_de, name, dtype):
     eager = make_runner(model, num_pages=32, page_size=64, max_requests=8)
     graph = make_runner(model, num_pages=32, page_size=64, max_requests=8, enable_graph=True)
     graph.graph_after = 1
+    graph.graph_mixed_pad_share = 0   # these small steps are recorded however many rows fill their shapes up
     rng = random.Random(3)
     n_max = min(cfg["max_position_embeddings"], 200)
     toks = {f"r{i}": random_tokens(cfg, rng.randint(30, n_max), 700 + i) for i in range(7)}
@@ -912,6 +913,19 @@ def test_recorded_steps_with_portions_of_prompts(models_de, name, dtype):
         for pos, row in logits[r]:
             assert rel_err(row[None], want[pos][None]) < TOL[dtype] * (1 if dtype == "bfloat16" else 5), f"{r} position {pos}"
     assert eager.cache.free_pages() == graph.cache.free_pages() == 32
+    # by default a step whose shape would be filled up by more than an eighth runs eagerly: 36 tokens would run as 48 rows
+    graph.graph_mixed_pad_share = 8
+    n_before = len(graph._graphs)
+    late = random_tokens(cfg, 66, 999)
+    assert cfg["max_position_embeddings"] >= 66
+    for run in (eager, graph):
+        run.cache.admit("late")
+    es = [StepEntry("late", late[:36], [35])]
+    assert torch.equal(eager.step(es), graph.step(es)) or dtype == "bfloat16"
+    assert len(graph._graphs) == n_before
+    es = [StepEntry("late", late[36:], [29])]      # 30 tokens run as 32 rows
+    graph.step(es)
+    assert len(graph._graphs) == n_before + 1
 
 
 @pytest.fixture(scope="module")
