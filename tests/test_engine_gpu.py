@@ -743,6 +743,52 @@ def _both_dtypes(cfg, num_pages, _unused=None):
         torch.cuda.empty_cache()
 
 
+@pytest.mark.parametrize("requests", [20, 40, 100, 150])
+def test_decode_steps_of_many_requests_at_the_8b_shape(requests):
+    """Two layers of the 8B shape in bfloat16 with 20 to 150 live requests of different lengths: their prompts in one
+    step, then decode steps that replay a recording of 24, 48, 128 or 160 rows (the products that keep chunks of X in
+    LDS with 2, 3, 8 and 10 groups of rows, the fragment-order q/k/v product up to 64 rows, the add+RMSNorm over many
+    float parts, attention chunks chosen by rounds of workgroups).  The decoded tokens' logits of a sample of the
+    requests against the plain implementation in float64 on the same weights."""
+    from infinilm_amd.engine.loading import build_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+    from infinilm_amd.weights import fill_random_
+
+    cfg = _real_shape("8b")
+    model = build_model(cfg, "bfloat16", "cuda:0")
+    fill_random_(model, seed=1, std=0.02, norm_init="one_plus")
+    r = make_runner(model, num_pages=2 * requests + 4, page_size=64, max_requests=requests, enable_graph=True)
+    r.graph_after = 1
+    g = torch.Generator().manual_seed(11 + requests)
+    lens = torch.randint(20, 90, (requests,), generator=g).tolist()
+    toks = [torch.randint(0, cfg["vocab_size"], (n + 3,), generator=g).tolist() for n in lens]
+    ids = [f"q{i}" for i in range(requests)]
+    for rid in ids:
+        r.cache.admit(rid)
+    r.step([StepEntry(rid, t[:n], []) for rid, t, n in zip(ids, toks, lens)])
+    got = []
+    for k in range(3):
+        got.append(r.step([StepEntry(rid, [t[n + k]], [0]) for rid, t, n in zip(ids, toks, lens)]).float().cpu().clone())
+    assert any(key[0] != "mixed" and key[0] == kernels_bound_rows(requests) for key in r._graphs), list(r._graphs)
+    W = {n: p.tensor.to(torch.float32) for n, p in model.named_parameters().items()}
+    sample = sorted(set([0, 1, requests // 2, requests - 2, requests - 1] + [int(i) for i in torch.randint(0, requests, (3,), generator=g)]))
+    worst = 0.0
+    for i in sample:
+        full = P.plain_forward(cfg, W, toks[i])
+        for k in range(3):
+            worst = max(worst, rel_err(got[k][i][None], full[lens[i] + k][None].cpu()))
+    print(f"[err] {requests} requests at the 8B shape: {worst:.3e}")
+    assert worst < TOL["bfloat16"], f"{requests} requests: {worst:.3e}"
+    for rid in ids:
+        r.cache.release(rid)
+    r.cache.check()
+
+
+def kernels_bound_rows(n):
+    from infinilm_amd import kernels
+    return kernels.bound_rows(n)
+
+
 def test_mixed_steps_at_the_8b_head_shape_with_recorded_steps_and_pages_used_again():
     """Two layers of the 8B shape (heads of 128 in groups of 16, pages of 64): five requests over a pool of 13
     pages, up to four live.  One step holds a portion with history, two decoded tokens and a fresh prompt
